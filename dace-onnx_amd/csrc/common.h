@@ -1,0 +1,102 @@
+// Shared device/host helpers for the gfx950 kernels of libmi355x_onnx.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/mi355x_onnx.h"
+
+namespace mi355x {
+
+// ---- host side: per-thread error channel -----------------------------------
+int set_error(int code, const char* fmt, ...);
+int check_launch(const char* kernel_name);
+
+#define MI355X_REQUIRE(cond, ...)                                              \
+    do {                                                                       \
+        if (!(cond)) return ::mi355x::set_error(MI355X_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- device side -------------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int WAVE = 64;  // CDNA wavefront width
+
+// DPP lane permutations inside a 16-lane row (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+constexpr int DPP_QUAD_XOR1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141; // lane i <-> 7-i inside 8 lanes
+constexpr int DPP_ROW_MIRROR = 0x140;      // lane i <-> 15-i inside 16 lanes
+
+__device__ __forceinline__ float readlane_f32(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// After row16_*: every lane holds the reduction over its 16-lane DPP row.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f32<DPP_QUAD_XOR1>(v);
+    v += dpp_f32<DPP_QUAD_XOR2>(v);
+    v += dpp_f32<DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f32<DPP_ROW_MIRROR>(v);
+    return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_f32<DPP_QUAD_XOR1>(v));
+    v = fmaxf(v, dpp_f32<DPP_QUAD_XOR2>(v));
+    v = fmaxf(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_f32<DPP_ROW_MIRROR>(v));
+    return v;
+}
+// Reduction over 32 lanes (lanes 0-31 and 32-63 each get their own result).
+__device__ __forceinline__ float half32_sum(float v) {
+    v = row16_sum(v);
+    const int base = (int)(threadIdx.x & 32);
+    // the two rows of this half: lanes base and base+16 hold the row totals
+    float lo = readlane_f32(v, 0), hi = readlane_f32(v, 16);
+    float lo2 = readlane_f32(v, 32), hi2 = readlane_f32(v, 48);
+    return base ? (lo2 + hi2) : (lo + hi);
+}
+__device__ __forceinline__ float half32_max(float v) {
+    v = row16_max(v);
+    const int base = (int)(threadIdx.x & 32);
+    float lo = readlane_f32(v, 0), hi = readlane_f32(v, 16);
+    float lo2 = readlane_f32(v, 32), hi2 = readlane_f32(v, 48);
+    return base ? fmaxf(lo2, hi2) : fmaxf(lo, hi);
+}
+// Reduction over the whole 64-lane wave; result is wave-uniform.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return (readlane_f32(v, 0) + readlane_f32(v, 16)) + (readlane_f32(v, 32) + readlane_f32(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(readlane_f32(v, 0), readlane_f32(v, 16)),
+                 fmaxf(readlane_f32(v, 32), readlane_f32(v, 48)));
+}
+
+// exact-erf Gelu, same formula as the exporter's Div, Erf, Add, Mul, Mul chain
+__device__ __forceinline__ float gelu_erf(float v) {
+    return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+}
+
+__device__ __forceinline__ float apply_epilogue(float v, int epi, float bias_v) {
+    if (epi & MI355X_EPI_BIAS) v += bias_v;
+    if (epi & MI355X_EPI_RELU) v = fmaxf(v, 0.0f);
+    if (epi & MI355X_EPI_GELU) v = gelu_erf(v);
+    return v;
+}
+
+}  // namespace mi355x

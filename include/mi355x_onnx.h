@@ -1,0 +1,168 @@
+/*
+ * mi355x_onnx.h -- C ABI of libmi355x_onnx.so: hand-written gfx950 (MI355X)
+ * kernels for the ONNX library nodes that DaCeML expands
+ * (MatMul/Gemm, Conv, MatMulInteger, Softmax, LayerNormalization,
+ * Add/Relu/Gelu and the Transpose copy that sits between them).
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is
+ *     allocated, freed or retained by the library (reference ownership rule:
+ *     daceml/pytorch/module_codegen.py:74-84,143-145 -- inputs are
+ *     .contiguous() data_ptr()s, outputs are pre-allocated by the caller);
+ *   - shapes and strides are int64 ELEMENT counts (not bytes);
+ *   - `stream` is a hipStream_t passed as void*; kernels are enqueued on it
+ *     and the call returns without synchronising (reference threading rule:
+ *     daceml/pytorch/module_codegen.py:461-463 sets state.nosync = True and
+ *     daceml/onnx/environments/cudnn.py:44 binds __dace_current_stream);
+ *   - return value 0 = enqueued; non-zero = nothing was launched and
+ *     mi355x_last_error() holds a message for the calling thread
+ *     (the reference's vendor-library glue prints and continues,
+ *     daceml/onnx/include/daceml_cudnn.h:15-22, or prints and exit(1)s,
+ *     daceml/onnx/include/dace_onnx.h:7-15; here the caller decides).
+ *
+ * A DaCe C++ tasklet links this library the way cuDNN is linked in
+ * daceml/onnx/environments/cudnn.py:11-67; Python loads it with ctypes the way
+ * the reference loads its ORT bridge (daceml/ort_api/raw_api_bindings.py:305-321).
+ */
+#ifndef MI355X_ONNX_H
+#define MI355X_ONNX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355X_ONNX_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* status codes */
+#define MI355X_OK 0
+#define MI355X_ERR_INVALID_ARGUMENT 1 /* shape/stride/attribute outside what the kernel supports */
+#define MI355X_ERR_LAUNCH 2           /* hipLaunchKernel reported an error */
+#define MI355X_ERR_NOT_INITIALIZED 3  /* no gfx950 device / runtime not usable */
+
+/* Library identity and error channel.
+ * Counterpart of the per-process handle object of the reference's cuDNN glue
+ * (daceml/onnx/include/daceml_cudnn.h:38-64): there is no handle here, the
+ * only per-thread state is the last error string. */
+int mi355x_version(void);
+const char* mi355x_last_error(void);
+
+/* Number of compute units of the current device (0 when no device is usable).
+ * Used by callers that size grids or report occupancy; no reference counterpart. */
+int mi355x_device_cu_count(void);
+
+/* ---- epilogue flags shared by GEMM and Conv (bitwise OR) ------------------
+ * Applied per output element in this order:
+ *   v = alpha * acc; if BIAS v += bias[n]; if RELU v = max(v,0);
+ *   if GELU v = 0.5*v*(1+erf(v/sqrt(2))); if RESIDUAL v += residual[m,n].
+ * Replaces the separate Add / Relu / (Div,Erf,Add,Mul,Mul) nodes that follow a
+ * contraction in the reference's graphs (daceml/onnx/op_implementations/
+ * pure_implementations.py:77-79,112-127,462-474); the reference fuses only by
+ * graph transformation (daceml/transformation/tasklet_fusion.py:35). */
+#define MI355X_EPI_NONE 0
+#define MI355X_EPI_BIAS 1
+#define MI355X_EPI_RELU 2
+#define MI355X_EPI_GELU 4
+#define MI355X_EPI_RESIDUAL 8
+
+/* ONNX MatMul / Gemm, fp32, on MFMA.
+ *   C[b0,b1,m,n] = epilogue(alpha * sum_k A[b0,b1,m,k] * B[b0,b1,k,n])
+ * Replaces PureMatMul.forward -> PureEinsum.forward -> DaCe BLAS node
+ * (daceml/onnx/op_implementations/pure_implementations.py:130-267) and
+ * PureGemm.forward (pure_implementations.py:433-459, transB=1 is expressed by
+ * swapping the two B strides).
+ *   a_strides = {batch0, batch1, m, k}; b_strides = {batch0, batch1, k, n};
+ *   c_strides = {batch0, batch1, m} (n stride is 1); r_strides like c_strides
+ *   for `residual` (ignored unless MI355X_EPI_RESIDUAL). A batch stride of 0
+ *   broadcasts that operand (numpy broadcasting of leading dims,
+ *   pure_implementations.py:189-208). Two batch levels let a head split/merge
+ *   ([B,S,H*D] <-> [B,H,S,D]) be expressed as strides instead of the
+ *   Reshape+Transpose copies of pure_implementations.py:369-379,477-513.
+ *   bias is [N] (ignored unless MI355X_EPI_BIAS). */
+int mi355x_gemm_f32(const float* A, const float* B, float* C,
+                    const float* bias, const float* residual,
+                    int64_t batch0, int64_t batch1,
+                    int64_t M, int64_t N, int64_t K,
+                    const int64_t* a_strides, const int64_t* b_strides,
+                    const int64_t* c_strides, const int64_t* r_strides,
+                    float alpha, int epilogue, void* stream);
+
+/* ONNX Conv, 2-D, NCHW, group 1, fp32, implicit GEMM on MFMA.
+ *   Y[n,m,oy,ox] = epilogue(sum_{c,r,s} W[m,c,r,s] *
+ *        X[n,c,oy*stride_h - pad_top + r*dil_h, ox*stride_w - pad_left + s*dil_w])
+ * with out-of-range X taken as 0. Replaces PureConv2D
+ * (daceml/onnx/op_implementations/img_op_implementations.py:164-326; that
+ * expansion requires zero pads and drops the stride term at :278,:291) and the
+ * cudnnConvolutionForward call of cudnn_implementations.py:303-322.
+ *   pads = {top, left, bottom, right} (ONNX order), strides = {h, w},
+ *   dilations = {h, w}. X, W, Y are C-contiguous; bias is [M] or NULL.
+ *   epilogue accepts MI355X_EPI_BIAS and MI355X_EPI_RELU. */
+int mi355x_conv2d_f32(const float* X, const float* W, const float* bias, float* Y,
+                      int64_t N, int64_t C, int64_t H, int64_t Wd,
+                      int64_t M, int64_t KH, int64_t KW,
+                      const int64_t* pads, const int64_t* strides,
+                      const int64_t* dilations, int epilogue, void* stream);
+
+/* ONNX MatMulInteger, int8 x int8 -> int32 on int8 MFMA, bit-exact.
+ *   Y[m,n] = sum_k (A[m,k] - a_zero_point) * (B[k,n] - b_zero_point)
+ * The reference has no expansion of its own for this node: the generated class
+ * (daceml/onnx/nodes/onnx_op.py:623-640) only has the "onnxruntime"
+ * implementation (onnx_op.py:686-687 -> node_codegen.py:321-573).
+ * A is [M,K], B is [K,N], Y is [M,N], all C-contiguous; zero points are
+ * scalars passed by value. */
+int mi355x_matmul_integer_i8(const int8_t* A, const int8_t* B,
+                             int32_t a_zero_point, int32_t b_zero_point,
+                             int32_t* Y, int64_t M, int64_t N, int64_t K,
+                             void* stream);
+
+/* ONNX Softmax along one axis, fp32. X viewed as [outer, axis_len, inner]
+ * (C-contiguous): y = exp(x - max) / sum(exp(x - max)) over axis_len.
+ * Replaces the five maps of PureSoftmax.forward
+ * (pure_implementations.py:346-366) with one pass. inner == 1 is the
+ * last-axis case. */
+int mi355x_softmax_f32(const float* X, float* Y,
+                       int64_t outer, int64_t axis_len, int64_t inner,
+                       void* stream);
+
+/* ONNX LayerNormalization over the last axis, fp32, X is [rows, cols]:
+ *   y = (x - mean) / sqrt(var + eps) * gamma + beta, biased variance.
+ * The reference has no such node (opset 12); it runs the exporter's
+ * decomposition ReduceMean, Sub, Pow, ReduceMean, Add, Sqrt, Div, Mul, Add
+ * (pure_implementations.py:97-109,82-84,59-74,77-79,41-56,92-94).
+ * gamma/beta are [cols]; beta may be NULL. */
+int mi355x_layernorm_f32(const float* X, const float* gamma, const float* beta,
+                         float* Y, int64_t rows, int64_t cols, float eps,
+                         void* stream);
+
+/* Elementwise ops, fp32, with numpy broadcasting.
+ * Replaces the one-map expansions Add/Sub/Mul/Div
+ * (pure_implementations.py:77-94), PureRelu (:462-474), PureErf (:112-127),
+ * PureSqrt (:41-56) and the Gelu decomposition Div,Erf,Add,Mul,Mul.
+ *   binary ops: C = A op B; unary ops ignore B (pass NULL).
+ *   ndim <= 8; shape is the OUTPUT shape; a_strides / b_strides are element
+ *   strides of each operand in the output's index space (0 on broadcast dims).
+ *   C is C-contiguous. */
+#define MI355X_OP_ADD 0
+#define MI355X_OP_SUB 1
+#define MI355X_OP_MUL 2
+#define MI355X_OP_DIV 3
+#define MI355X_OP_RELU 16
+#define MI355X_OP_GELU 17
+#define MI355X_OP_ERF 18
+#define MI355X_OP_SQRT 19
+int mi355x_eltwise_f32(int op, const float* A, const float* B, float* C,
+                       int ndim, const int64_t* shape,
+                       const int64_t* a_strides, const int64_t* b_strides,
+                       void* stream);
+
+/* ONNX Transpose (and any strided gather), 4-byte elements:
+ *   Y (C-contiguous, `shape`) [i0..] = X[sum_d i_d * x_strides[d]].
+ * Replaces PureTranspose.forward (pure_implementations.py:369-379). ndim <= 8. */
+int mi355x_permute_b32(const void* X, void* Y, int ndim, const int64_t* shape,
+                       const int64_t* x_strides, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_ONNX_H */
