@@ -33,7 +33,7 @@ namespace mi355x {
 struct MMIArgs {
     const int8_t* A; const int8_t* B; int32_t* Y;
     int64_t M, N, K;
-    int32_t za, zb;
+    const int8_t* za_ptr; const int8_t* zb_ptr;
     int64_t tiles_m, tiles_n, nwg;
 };
 
@@ -148,7 +148,9 @@ __global__ __launch_bounds__(256) void matmul_integer_i8_kernel(MMIArgs p) {
             for (int r = 0; r < 16; ++r) acc[i][t][r] = 0;
     int32_t rowsum[2] = {0, 0};  // partial: rows wm0+32i+lj, this lane's k half
     int32_t colsum[2] = {0, 0};  // partial: cols wn0+2*lj+t, this lane's k half
-    const bool need_rowsum = p.zb != 0, need_colsum = p.za != 0;
+    // zero points are device scalars (wave-uniform loads); NULL means 0
+    const int32_t za_i = p.za_ptr ? (int32_t)*p.za_ptr : 0, zb_i = p.zb_ptr ? (int32_t)*p.zb_ptr : 0;
+    const bool need_rowsum = zb_i != 0, need_colsum = za_i != 0;
 
     const int64_t ktiles = (p.K + BK - 1) / BK;
     load_tiles(0);
@@ -209,7 +211,7 @@ __global__ __launch_bounds__(256) void matmul_integer_i8_kernel(MMIArgs p) {
     }
     __syncthreads();
 
-    const uint32_t za = (uint32_t)p.za, zb = (uint32_t)p.zb;
+    const uint32_t za = (uint32_t)za_i, zb = (uint32_t)zb_i;
     const uint32_t kzz = (uint32_t)p.K * za * zb;
     // acc[i][t][r] = Y[m0+wm0+32i + 8*(r/4)+4*lg+(r%4)][n0+wn0+2*lj+t]
     const int64_t n = n0 + wn0 + 2 * lj;
@@ -237,19 +239,17 @@ __global__ __launch_bounds__(256) void matmul_integer_i8_kernel(MMIArgs p) {
 
 }  // namespace mi355x
 
-extern "C" int mi355x_matmul_integer_i8(const int8_t* A, const int8_t* B, int32_t a_zero_point,
-                                        int32_t b_zero_point, int32_t* Y, int64_t M, int64_t N,
-                                        int64_t K, void* stream) {
+extern "C" int mi355x_matmul_integer_i8(const int8_t* A, const int8_t* B,
+                                        const int8_t* a_zero_point, const int8_t* b_zero_point,
+                                        int32_t* Y, int64_t M, int64_t N, int64_t K, void* stream) {
     using namespace mi355x;
     MI355X_REQUIRE(M >= 0 && N >= 0 && K >= 0, "matmul_integer: negative extent (M=%lld N=%lld K=%lld)",
                    (long long)M, (long long)N, (long long)K);
-    MI355X_REQUIRE(a_zero_point >= -128 && a_zero_point <= 127 && b_zero_point >= -128 && b_zero_point <= 127,
-                   "matmul_integer: zero points (%d, %d) outside int8", a_zero_point, b_zero_point);
     if (M == 0 || N == 0) return MI355X_OK;
     MI355X_REQUIRE(A && B && Y, "matmul_integer: null pointer");
     MMIArgs p;
     p.A = A; p.B = B; p.Y = Y; p.M = M; p.N = N; p.K = K;
-    p.za = a_zero_point; p.zb = b_zero_point;
+    p.za_ptr = a_zero_point; p.zb_ptr = b_zero_point;
     p.tiles_m = ceil_div(M, MMI_BM);
     p.tiles_n = ceil_div(N, MMI_BN);
     p.nwg = p.tiles_m * p.tiles_n;

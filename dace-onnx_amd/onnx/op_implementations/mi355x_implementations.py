@@ -1,0 +1,561 @@
+"""The ``"mi355x"`` expansions: ONNX library nodes -> calls into libmi355x_onnx.so.
+
+Each class has the shape of a reference expansion (``ONNXForward`` with
+``forward_can_be_applied`` / ``forward``, registered through
+``op_implementation(op=..., name="mi355x")``) and stands where the reference has
+its ``"pure"`` / ``"cuDNN"`` classes:
+
+==================  ============================================================
+MatMul              PureMatMul -> PureEinsum, pure_implementations.py:130-267
+Gemm                PureGemm, pure_implementations.py:433-459
+Conv                PureConv2D, img_op_implementations.py:164-326;
+                    CudnnConvolution, cudnn_implementations.py:111-336
+MatMulInteger       (ONNX Runtime only, onnx_op.py:686-687)
+Softmax             PureSoftmax, pure_implementations.py:346-366
+LayerNormalization  (exporter decomposition, pure_implementations.py:97-109 etc.)
+Add/Sub/Mul/Div     python_pure_op_implementation, pure_implementations.py:77-94
+Relu, Erf, Sqrt     pure_implementations.py:462-474, 112-127, 41-56
+Gelu                (exporter decomposition Div, Erf, Add, Mul, Mul)
+Transpose           PureTranspose, pure_implementations.py:369-379
+Reshape, Flatten    PureReshape / PureFlatten, pure_implementations.py:477-526
+Identity            pure_implementations.py:270-272
+==================  ============================================================
+
+``forward_can_be_applied`` mirrors every precondition of the kernel it would
+call, so an unsupported configuration is refused before anything is launched
+(and, there being no ONNX Runtime here, reported as an error by the fallback).
+``forward`` returns a :class:`~dace_onnx_amd.sdfg.KernelCall`.
+"""
+import typing
+
+import numpy as np
+
+from ... import sdfg as dace
+from ... import _lib
+from ...sdfg import SDFG, SDFGState, Ptr, Stream, I64Array, AliasNode
+from ...util.utils import in_desc_with_name, out_desc_with_name, prod
+from ..forward_implementation_abc import ONNXForward
+from .utils import op_implementation, kernel_call_for_node
+
+IMPLEMENTATION_NAME = "mi355x"
+MAX_ELTWISE_DIMS = 8
+
+
+def _is_f32(*descs) -> bool:
+    return all(d.dtype == dace.float32 for d in descs)
+
+
+def _contig(*descs) -> bool:
+    return all(d.is_contiguous() for d in descs)
+
+
+def _has_input(node, state, name) -> bool:
+    return any(e.dst_conn == name for e in state.in_edges(node))
+
+
+def _has_output(node, state, name) -> bool:
+    return any(e.src_conn == name for e in state.out_edges(node))
+
+
+def _broadcast_shape(*shapes):
+    try:
+        return tuple(np.broadcast_shapes(*shapes))
+    except ValueError:
+        return None
+
+
+def _broadcast_strides(desc, out_shape):
+    """Element strides of ``desc`` in the index space of ``out_shape`` (0 where broadcast)."""
+    pad = len(out_shape) - len(desc.shape)
+    strides = []
+    for d, extent in enumerate(out_shape):
+        if d < pad or desc.shape[d - pad] == 1:
+            strides.append(0)
+        else:
+            strides.append(desc.strides[d - pad])
+    return strides
+
+
+# ------------------------------------------------------------------------------------
+# contractions
+
+
+class _BatchPlan:
+    """How a numpy-style batched matmul maps onto the kernel's two batch levels."""
+
+    def __init__(self, A, B, Y):
+        self.ok = False
+        if len(A.shape) < 2 or len(B.shape) < 2:
+            return
+        M, K = A.shape[-2:]
+        K2, N = B.shape[-2:]
+        if K != K2:
+            return
+        batch = _broadcast_shape(A.shape[:-2], B.shape[:-2])
+        if batch is None or tuple(Y.shape) != tuple(batch) + (M, N) or Y.strides[-1] != 1 and N != 1:
+            return
+        a_bs = _broadcast_strides(dace.Array(A.dtype, A.shape[:-2], A.strides[:-2]), batch)
+        b_bs = _broadcast_strides(dace.Array(B.dtype, B.shape[:-2], B.strides[:-2]), batch)
+        y_bs = list(Y.strides[:-2])
+        dims = [(e, a, b, y) for e, a, b, y in zip(batch, a_bs, b_bs, y_bs) if e != 1]
+        a_sm, a_sk = A.strides[-2:]
+        b_sk, b_sn = B.strides[-2:]
+        y_sm = Y.strides[-2]
+        # B shared by every batch entry: fold batch dims into M while A and Y allow it
+        while dims and dims[-1][2] == 0 and dims[-1][1] == M * a_sm and dims[-1][3] == M * y_sm:
+            M *= dims[-1][0]
+            dims.pop()
+        # merge adjacent batch dims that all three operands walk as one
+        merged = []
+        for d in dims:
+            if merged:
+                e0, a0, b0, y0 = merged[-1]
+                if a0 == d[1] * d[0] and b0 == d[2] * d[0] and y0 == d[3] * d[0]:
+                    merged[-1] = (e0 * d[0], d[1], d[2], d[3])
+                    continue
+            merged.append(d)
+        if len(merged) > 2:
+            return
+        while len(merged) < 2:
+            merged.insert(0, (1, 0, 0, 0))
+        (self.batch0, a0, b0, y0), (self.batch1, a1, b1, y1) = merged
+        self.M, self.N, self.K = M, N, K
+        self.a_strides = [a0, a1, a_sm, a_sk]
+        self.b_strides = [b0, b1, b_sk, b_sn]
+        self.c_strides = [y0, y1, y_sm]
+        self.ok = True
+
+
+def _gemm_call(node, state, plan, a_conn, b_conn, y_conn, bias_conn=None, residual_conn=None,
+               r_strides=None, alpha=1.0, epilogue=_lib.EPI_NONE):
+    return kernel_call_for_node(node, state, "mi355x_gemm_f32", [
+        Ptr(a_conn), Ptr(b_conn), Ptr(y_conn), Ptr(bias_conn), Ptr(residual_conn),
+        plan.batch0, plan.batch1, plan.M, plan.N, plan.K,
+        I64Array(plan.a_strides), I64Array(plan.b_strides), I64Array(plan.c_strides),
+        I64Array(r_strides) if r_strides is not None else None,
+        float(alpha), int(epilogue), Stream()])
+
+
+def _fused_epilogue(node, state, sdfg, plan):
+    """Epilogue requested by the fusion pass through private node attributes
+    (the reference passes per-node tuning the same way: ``node._algorithm``,
+    cudnn_implementations.py:251-254). Extra inputs use the connectors
+    ``_bias`` ([N]) and ``_residual`` (same shape as Y)."""
+    epi = 0
+    bias_conn = residual_conn = r_strides = None
+    if _has_input(node, state, "_bias"):
+        epi |= _lib.EPI_BIAS
+        bias_conn = "_bias"
+    act = getattr(node, "_activation", None)
+    if act == "relu":
+        epi |= _lib.EPI_RELU
+    elif act == "gelu":
+        epi |= _lib.EPI_GELU
+    if _has_input(node, state, "_residual"):
+        epi |= _lib.EPI_RESIDUAL
+        residual_conn = "_residual"
+        r = in_desc_with_name(node, state, sdfg, "_residual")
+        y = out_desc_with_name(node, state, sdfg, "Y")
+        if tuple(r.shape) != tuple(y.shape) or tuple(r.strides) != tuple(y.strides):
+            raise ValueError("fused residual must have the shape and layout of Y")
+        r_strides = plan.c_strides
+    return epi, bias_conn, residual_conn, r_strides
+
+
+@op_implementation(op="MatMul", name=IMPLEMENTATION_NAME)
+class MI355XMatMul(ONNXForward):
+    """numpy-style (batched, broadcasting) matmul on the fp32 MFMA GEMM kernel.
+    Leading dimensions become the kernel's batch levels, or part of M when B is
+    shared; nothing is copied or transposed."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        A = in_desc_with_name(node, state, sdfg, "A")
+        B = in_desc_with_name(node, state, sdfg, "B")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        if len(A.shape) == 1 or len(B.shape) == 1:  # same refusal as PureMatMul (:133-140)
+            return False
+        if not _is_f32(A, B, Y):
+            return False
+        return _BatchPlan(A, B, Y).ok
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        A = in_desc_with_name(node, state, sdfg, "A")
+        B = in_desc_with_name(node, state, sdfg, "B")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        a_view = getattr(node, "_a_view", None)  # (shape, strides) set by the fusion pass
+        b_view = getattr(node, "_b_view", None)
+        y_view = getattr(node, "_y_view", None)
+        if a_view:
+            A = dace.Array(A.dtype, *a_view)
+        if b_view:
+            B = dace.Array(B.dtype, *b_view)
+        if y_view:
+            Y = dace.Array(Y.dtype, *y_view)
+        plan = _BatchPlan(A, B, Y)
+        if not plan.ok:
+            raise ValueError(f"{node.label}: operand layout cannot be expressed as a strided batched GEMM")
+        epi, bias_conn, residual_conn, r_strides = _fused_epilogue(node, state, sdfg, plan)
+        return _gemm_call(node, state, plan, "A", "B", "Y", bias_conn, residual_conn, r_strides,
+                          alpha=getattr(node, "_alpha", 1.0), epilogue=epi)
+
+
+@op_implementation(op="Gemm", name=IMPLEMENTATION_NAME)
+class MI355XGemm(ONNXForward):
+    """``Y = alpha * A' B' + beta * C``. transA / transB are strides; ``C`` is
+    fused as a row bias (shape [N] or [1,N]) or as a full [M,N] addend.
+    PureGemm only accepts alpha=1, beta=1, transA=0, transB=1 (:436-440)."""
+
+    @staticmethod
+    def _c_kind(C, M, N):
+        if C is None:
+            return "none"
+        shape = tuple(C.shape)
+        if shape in ((N, ), (1, N)) and C.strides[-1] == 1:
+            return "bias"
+        if shape == (M, N) and C.strides[-1] == 1:
+            return "full"
+        return None
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        A = in_desc_with_name(node, state, sdfg, "A")
+        B = in_desc_with_name(node, state, sdfg, "B")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        C = in_desc_with_name(node, state, sdfg, "C") if _has_input(node, state, "C") else None
+        if len(A.shape) != 2 or len(B.shape) != 2 or len(Y.shape) != 2:
+            return False
+        if not _is_f32(A, B, Y) or (C is not None and not _is_f32(C)):
+            return False
+        M, K = (A.shape[1], A.shape[0]) if node.transA else A.shape
+        K2, N = (B.shape[1], B.shape[0]) if node.transB else B.shape
+        if K != K2 or tuple(Y.shape) != (M, N) or Y.strides[-1] != 1:
+            return False
+        if C is not None and node.beta not in (0.0, 1.0):
+            return False
+        if C is not None and node.beta == 1.0 and MI355XGemm._c_kind(C, M, N) is None:
+            return False
+        return True
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        A = in_desc_with_name(node, state, sdfg, "A")
+        B = in_desc_with_name(node, state, sdfg, "B")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        C = in_desc_with_name(node, state, sdfg, "C") if _has_input(node, state, "C") else None
+        if node.transA:
+            A = dace.Array(A.dtype, A.shape[::-1], A.strides[::-1])
+        if node.transB:
+            B = dace.Array(B.dtype, B.shape[::-1], B.strides[::-1])
+        plan = _BatchPlan(A, B, Y)
+        assert plan.ok
+        kind = MI355XGemm._c_kind(C, plan.M, plan.N) if (C is not None and node.beta == 1.0) else "none"
+        epi, bias_conn, residual_conn, r_strides = 0, None, None, None
+        if kind == "bias":
+            epi, bias_conn = _lib.EPI_BIAS, "C"
+        elif kind == "full":
+            epi, residual_conn, r_strides = _lib.EPI_RESIDUAL, "C", [0, 0, C.strides[0]]
+        act = getattr(node, "_activation", None)
+        if act == "relu":
+            epi |= _lib.EPI_RELU
+        elif act == "gelu":
+            epi |= _lib.EPI_GELU
+        return _gemm_call(node, state, plan, "A", "B", "Y", bias_conn, residual_conn, r_strides,
+                          alpha=float(node.alpha), epilogue=epi)
+
+
+def _conv_geometry(node, X, W):
+    """(pads[4], strides[2], dilations[2], out_h, out_w) under ONNX rules, or None."""
+    if len(X.shape) != 4 or len(W.shape) != 4:
+        return None
+    H, Wd = X.shape[2:]
+    KH, KW = W.shape[2:]
+    strides = list(node.strides) if node.strides is not None else [1, 1]
+    dil = list(node.dilations) if node.dilations is not None else [1, 1]
+    if len(strides) != 2 or len(dil) != 2 or min(strides + dil) < 1:
+        return None
+    if node.kernel_shape is not None and list(node.kernel_shape) != [KH, KW]:
+        return None
+    eff = [(KH - 1) * dil[0] + 1, (KW - 1) * dil[1] + 1]
+    auto_pad = node.auto_pad or "NOTSET"
+    if auto_pad == "NOTSET":
+        pads = list(node.pads) if node.pads is not None else [0, 0, 0, 0]
+        if len(pads) != 4 or min(pads) < 0:
+            return None
+    elif auto_pad == "VALID":
+        pads = [0, 0, 0, 0]
+    elif auto_pad in ("SAME_UPPER", "SAME_LOWER"):
+        pads = [0, 0, 0, 0]
+        for i, (size, s) in enumerate(((H, strides[0]), (Wd, strides[1]))):
+            out = -(-size // s)
+            total = max((out - 1) * s + eff[i] - size, 0)
+            lo = total // 2 if auto_pad == "SAME_UPPER" else total - total // 2
+            pads[i], pads[i + 2] = lo, total - lo
+    else:
+        return None
+    hin, win = H + pads[0] + pads[2], Wd + pads[1] + pads[3]
+    if hin < eff[0] or win < eff[1]:
+        return None
+    return pads, strides, dil, (hin - eff[0]) // strides[0] + 1, (win - eff[1]) // strides[1] + 1
+
+
+@op_implementation(op="Conv", name=IMPLEMENTATION_NAME)
+class MI355XConv(ONNXForward):
+    """2-D NCHW convolution as implicit GEMM on MFMA. Honours ``strides``,
+    ``pads`` (also asymmetric), ``dilations`` and ``auto_pad``; the bias and a
+    following Relu are applied in the kernel's epilogue. PureConv2D refuses any
+    non-zero pad and ignores the stride (img_op_implementations.py:201-203,278)."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "X")
+        W = in_desc_with_name(node, state, sdfg, "W")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        B = in_desc_with_name(node, state, sdfg, "B") if _has_input(node, state, "B") else None
+        if not _is_f32(X, W, Y) or not _contig(X, W, Y):
+            return False
+        if len(X.shape) != 4 or len(W.shape) != 4:  # only 2-D, like the pure and cuDNN versions
+            return False
+        if node.group != 1 or X.shape[1] != W.shape[1]:
+            return False
+        geom = _conv_geometry(node, X, W)
+        if geom is None:
+            return False
+        if tuple(Y.shape) != (X.shape[0], W.shape[0], geom[3], geom[4]):
+            return False
+        if B is not None and (not _is_f32(B) or tuple(B.shape) != (W.shape[0], ) or not _contig(B)):
+            return False
+        if prod(X.shape) >= 2**30 or prod(Y.shape) >= 2**31:
+            return False
+        return True
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "X")
+        W = in_desc_with_name(node, state, sdfg, "W")
+        has_bias = _has_input(node, state, "B")
+        pads, strides, dil, _, _ = _conv_geometry(node, X, W)
+        epi = (_lib.EPI_BIAS if has_bias else 0) | (_lib.EPI_RELU if getattr(node, "_activation", None) == "relu" else 0)
+        N, C, H, Wd = X.shape
+        M, _, KH, KW = W.shape
+        return kernel_call_for_node(node, state, "mi355x_conv2d_f32", [
+            Ptr("X"), Ptr("W"), Ptr("B" if has_bias else None), Ptr("Y"),
+            N, C, H, Wd, M, KH, KW, I64Array(pads), I64Array(strides), I64Array(dil), epi, Stream()])
+
+
+@op_implementation(op="MatMulInteger", name=IMPLEMENTATION_NAME)
+class MI355XMatMulInteger(ONNXForward):
+    """int8 x int8 -> int32 on int8 MFMA, bit-exact, scalar zero points read on
+    the device. The reference can only run this node through ONNX Runtime."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        A = in_desc_with_name(node, state, sdfg, "A")
+        B = in_desc_with_name(node, state, sdfg, "B")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        if A.dtype != dace.int8 or B.dtype != dace.int8 or Y.dtype != dace.int32:
+            return False
+        if len(A.shape) != 2 or len(B.shape) != 2 or A.shape[1] != B.shape[0]:
+            return False
+        if tuple(Y.shape) != (A.shape[0], B.shape[1]) or not _contig(A, B, Y):
+            return False
+        for zp in ("a_zero_point", "b_zero_point"):
+            if _has_input(node, state, zp):
+                d = in_desc_with_name(node, state, sdfg, zp)
+                if d.dtype != dace.int8 or d.total_size != 1:  # per-row / per-column zero points
+                    return False
+        return True
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        A = in_desc_with_name(node, state, sdfg, "A")
+        B = in_desc_with_name(node, state, sdfg, "B")
+        za = "a_zero_point" if _has_input(node, state, "a_zero_point") else None
+        zb = "b_zero_point" if _has_input(node, state, "b_zero_point") else None
+        return kernel_call_for_node(node, state, "mi355x_matmul_integer_i8", [
+            Ptr("A"), Ptr("B"), Ptr(za), Ptr(zb), Ptr("Y"), A.shape[0], B.shape[1], A.shape[1], Stream()])
+
+
+# ------------------------------------------------------------------------------------
+# row reductions
+
+
+@op_implementation(op="Softmax", name=IMPLEMENTATION_NAME)
+class MI355XSoftmax(ONNXForward):
+    """Softmax along ``node.axis`` only, the semantics of PureSoftmax
+    (:352-364; for the last axis this equals the opset-11 flattened form)."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "input")
+        Y = out_desc_with_name(node, state, sdfg, "output")
+        if not _is_f32(X, Y) or not _contig(X, Y) or tuple(X.shape) != tuple(Y.shape):
+            return False
+        return len(X.shape) >= 1 and -len(X.shape) <= node.axis < len(X.shape)
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "input")
+        axis = node.axis % len(X.shape)
+        outer, axis_len, inner = prod(X.shape[:axis]), X.shape[axis], prod(X.shape[axis + 1:])
+        return kernel_call_for_node(node, state, "mi355x_softmax_f32",
+                                    [Ptr("input"), Ptr("output"), outer, axis_len, inner, Stream()])
+
+
+@op_implementation(op="LayerNormalization", name=IMPLEMENTATION_NAME)
+class MI355XLayerNormalization(ONNXForward):
+    """One-pass layer normalization over the dimensions from ``axis`` on."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "X")
+        S = in_desc_with_name(node, state, sdfg, "Scale")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        descs = [X, S, Y]
+        if _has_input(node, state, "B"):
+            descs.append(in_desc_with_name(node, state, sdfg, "B"))
+        if not _is_f32(*descs) or not _contig(*descs) or tuple(X.shape) != tuple(Y.shape):
+            return False
+        if _has_output(node, state, "Mean") or _has_output(node, state, "InvStdDev"):
+            return False
+        if len(X.shape) < 1 or not (-len(X.shape) <= node.axis < len(X.shape)):
+            return False
+        cols = prod(X.shape[node.axis % len(X.shape):])
+        return all(d.total_size == cols for d in descs[1:2] + descs[3:])
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "X")
+        axis = node.axis % len(X.shape)
+        rows, cols = prod(X.shape[:axis]), prod(X.shape[axis:])
+        beta = "B" if _has_input(node, state, "B") else None
+        return kernel_call_for_node(node, state, "mi355x_layernorm_f32", [
+            Ptr("X"), Ptr("Scale"), Ptr(beta), Ptr("Y"), rows, cols, float(node.epsilon), Stream()])
+
+
+# ------------------------------------------------------------------------------------
+# elementwise
+
+
+def _binary_impl(op_name, opcode):
+    @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
+    class Impl(ONNXForward):
+        __doc__ = f"``C = A {op_name.lower()} B`` with numpy broadcasting, one pass."
+
+        @staticmethod
+        def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+            A = in_desc_with_name(node, state, sdfg, "A")
+            B = in_desc_with_name(node, state, sdfg, "B")
+            C = out_desc_with_name(node, state, sdfg, "C")
+            if not _is_f32(A, B, C) or not _contig(C):
+                return False
+            out = _broadcast_shape(A.shape, B.shape)
+            return out is not None and tuple(C.shape) == out and len(out) <= MAX_ELTWISE_DIMS
+
+        @staticmethod
+        def forward(node, state: SDFGState, sdfg: SDFG):
+            A = in_desc_with_name(node, state, sdfg, "A")
+            B = in_desc_with_name(node, state, sdfg, "B")
+            C = out_desc_with_name(node, state, sdfg, "C")
+            return kernel_call_for_node(node, state, "mi355x_eltwise_f32", [
+                opcode, Ptr("A"), Ptr("B"), Ptr("C"), len(C.shape), I64Array(C.shape),
+                I64Array(_broadcast_strides(A, C.shape)), I64Array(_broadcast_strides(B, C.shape)), Stream()])
+
+    Impl.__name__ = Impl.__qualname__ = "MI355X" + op_name
+    return Impl
+
+
+MI355XAdd = _binary_impl("Add", _lib.OP_ADD)
+MI355XSub = _binary_impl("Sub", _lib.OP_SUB)
+MI355XMul = _binary_impl("Mul", _lib.OP_MUL)
+MI355XDiv = _binary_impl("Div", _lib.OP_DIV)
+
+
+def _unary_impl(op_name, opcode, in_conn, out_conn, extra_check=None):
+    @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
+    class Impl(ONNXForward):
+        __doc__ = f"Elementwise {op_name}, one pass, 16 bytes per lane."
+
+        @staticmethod
+        def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+            X = in_desc_with_name(node, state, sdfg, in_conn)
+            Y = out_desc_with_name(node, state, sdfg, out_conn)
+            if not _is_f32(X, Y) or not _contig(X, Y) or tuple(X.shape) != tuple(Y.shape):
+                return False
+            return extra_check(node) if extra_check else True
+
+        @staticmethod
+        def forward(node, state: SDFGState, sdfg: SDFG):
+            X = in_desc_with_name(node, state, sdfg, in_conn)
+            return kernel_call_for_node(node, state, "mi355x_eltwise_f32", [
+                opcode, Ptr(in_conn), None, Ptr(out_conn), 1, I64Array([X.total_size]), I64Array([1]),
+                None, Stream()])
+
+    Impl.__name__ = Impl.__qualname__ = "MI355X" + op_name
+    return Impl
+
+
+MI355XRelu = _unary_impl("Relu", _lib.OP_RELU, "X", "Y")
+MI355XGelu = _unary_impl("Gelu", _lib.OP_GELU, "X", "Y",
+                         extra_check=lambda node: (node.approximate or "none") == "none")
+MI355XErf = _unary_impl("Erf", _lib.OP_ERF, "input", "output")
+MI355XSqrt = _unary_impl("Sqrt", _lib.OP_SQRT, "X", "Y")
+
+
+# ------------------------------------------------------------------------------------
+# data movement
+
+
+@op_implementation(op="Transpose", name=IMPLEMENTATION_NAME)
+class MI355XTranspose(ONNXForward):
+    """Permutation copy for 4-byte element types."""
+
+    @staticmethod
+    def _perm(node, rank):
+        return list(node.perm) if node.perm is not None else list(reversed(range(rank)))
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "data")
+        Y = out_desc_with_name(node, state, sdfg, "transposed")
+        if X.dtype != Y.dtype or X.dtype.bytes != 4 or not _contig(Y) or len(X.shape) > MAX_ELTWISE_DIMS:
+            return False
+        perm = MI355XTranspose._perm(node, len(X.shape))
+        if sorted(perm) != list(range(len(X.shape))):
+            return False
+        return tuple(Y.shape) == tuple(X.shape[p] for p in perm)
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "data")
+        perm = MI355XTranspose._perm(node, len(X.shape))
+        return kernel_call_for_node(node, state, "mi355x_permute_b32", [
+            Ptr("data"), Ptr("transposed"), len(perm), I64Array([X.shape[p] for p in perm]),
+            I64Array([X.strides[p] for p in perm]), Stream()])
+
+
+def _alias_impl(op_name, in_conn, out_conn):
+    @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
+    class Impl(ONNXForward):
+        __doc__ = (f"{op_name} of contiguous data is a view: the output aliases the input's storage. "
+                   "(PureReshape copies through ``np.reshape``, pure_implementations.py:496-513; "
+                   "like it, the constant ``shape`` input is dropped.)")
+
+        @staticmethod
+        def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+            X = in_desc_with_name(node, state, sdfg, in_conn)
+            Y = out_desc_with_name(node, state, sdfg, out_conn)
+            return X.dtype == Y.dtype and _contig(X, Y) and X.total_size == Y.total_size
+
+        @staticmethod
+        def forward(node, state: SDFGState, sdfg: SDFG):
+            return AliasNode(node.label + "_view", in_conn, out_conn)
+
+    Impl.__name__ = Impl.__qualname__ = "MI355X" + op_name
+    return Impl
+
+
+MI355XReshape = _alias_impl("Reshape", "data", "reshaped")
+MI355XFlatten = _alias_impl("Flatten", "input", "output")
+MI355XIdentity = _alias_impl("Identity", "input", "output")

@@ -1,0 +1,131 @@
+"""Static shape and type inference for the supported ops.
+
+The reference runs ``onnx.shape_inference`` (or the vendored symbolic inference,
+``daceml/onnx/shape_inference/symbolic_shape_infer.py``) before it creates one
+array per value (``daceml/onnx/onnx_importer.py:131-166``). Shapes on the hot
+path are static, so this is the per-op rule set of the ONNX specification for
+the ops that have an ``ONNX<Op>`` class here; value_info already present in the
+model is kept and checked against.
+"""
+import typing
+
+import numpy as np
+
+from .proto import ModelProto, ValueInfoProto, TensorProto, np_dtype_to_tensor_dtype
+
+
+class ShapeInferenceError(ValueError):
+    pass
+
+
+def _attrs(node):
+    return {a.name: a.value for a in node.attribute}
+
+
+def _conv_out(size, k, stride, dil, pad_lo, pad_hi):
+    return (size + pad_lo + pad_hi - ((k - 1) * dil + 1)) // stride + 1
+
+
+def _infer_node(node, shapes, types, constants):
+    """Return [(shape, elem_type)] for each output of ``node``."""
+    a = _attrs(node)
+    ins = [shapes.get(i) for i in node.input]
+    tys = [types.get(i) for i in node.input]
+    op = node.op_type
+    if any(s is None for s, name in zip(ins, node.input) if name != ""):
+        missing = [n for n in node.input if n and n not in shapes]
+        raise ShapeInferenceError(f"{op} node '{node.name}': no shape for input(s) {missing}")
+    if op in ("Add", "Sub", "Mul", "Div", "Pow"):
+        return [(tuple(np.broadcast_shapes(ins[0], ins[1])), tys[0])]
+    if op in ("Relu", "Gelu", "Erf", "Sqrt", "Softmax", "Identity", "Tanh", "Sigmoid"):
+        return [(ins[0], tys[0])]
+    if op == "LayerNormalization":
+        return [(ins[0], tys[0])]
+    if op == "MatMul" or op == "MatMulInteger":
+        A, B = ins[0], ins[1]
+        if len(A) < 2 or len(B) < 2:
+            raise ShapeInferenceError(f"{op} '{node.name}': 1-D operands are not supported")
+        if A[-1] != B[-2]:
+            raise ShapeInferenceError(f"{op} '{node.name}': inner dimensions {A[-1]} and {B[-2]} differ")
+        batch = tuple(np.broadcast_shapes(A[:-2], B[:-2]))
+        return [(batch + (A[-2], B[-1]), TensorProto.INT32 if op == "MatMulInteger" else tys[0])]
+    if op == "Gemm":
+        A, B = ins[0], ins[1]
+        M = A[1] if a.get("transA", 0) else A[0]
+        N = B[0] if a.get("transB", 0) else B[1]
+        return [((M, N), tys[0])]
+    if op == "Conv":
+        X, W = ins[0], ins[1]
+        nsp = len(X) - 2
+        strides = a.get("strides") or [1] * nsp
+        dil = a.get("dilations") or [1] * nsp
+        auto_pad = a.get("auto_pad", "NOTSET")
+        if isinstance(auto_pad, bytes):
+            auto_pad = auto_pad.decode()
+        out = []
+        for i in range(nsp):
+            if auto_pad in ("SAME_UPPER", "SAME_LOWER"):
+                out.append(-(-X[2 + i] // strides[i]))
+            else:
+                pads = (a.get("pads") or [0] * (2 * nsp)) if auto_pad == "NOTSET" else [0] * (2 * nsp)
+                out.append(_conv_out(X[2 + i], W[2 + i], strides[i], dil[i], pads[i], pads[i + nsp]))
+        return [((X[0], W[0]) + tuple(out), tys[0])]
+    if op == "Transpose":
+        perm = a.get("perm") or list(reversed(range(len(ins[0]))))
+        return [(tuple(ins[0][p] for p in perm), tys[0])]
+    if op == "Reshape":
+        if node.input[1] not in constants:
+            raise ShapeInferenceError(f"Reshape '{node.name}': the shape input must be a constant initializer")
+        target = [int(v) for v in constants[node.input[1]].ravel()]
+        total = int(np.prod(ins[0])) if len(ins[0]) else 1
+        out = [ins[0][i] if v == 0 else v for i, v in enumerate(target)]
+        if out.count(-1) > 1:
+            raise ShapeInferenceError(f"Reshape '{node.name}': more than one -1 in {target}")
+        if -1 in out:
+            known = int(np.prod([v for v in out if v != -1])) if len(out) > 1 else 1
+            out[out.index(-1)] = total // known if known else 0
+        if int(np.prod(out)) != total:
+            raise ShapeInferenceError(f"Reshape '{node.name}': cannot reshape {ins[0]} to {target}")
+        return [(tuple(out), tys[0])]
+    if op == "Flatten":
+        axis = a.get("axis", 1) % (len(ins[0]) + 1) if a.get("axis", 1) < 0 else a.get("axis", 1)
+        return [((int(np.prod(ins[0][:axis])) if axis else 1, int(np.prod(ins[0][axis:]))), tys[0])]
+    if op == "ReduceMean":
+        axes = a.get("axes") or list(range(len(ins[0])))
+        axes = [ax % len(ins[0]) for ax in axes]
+        keep = a.get("keepdims", 1)
+        out = [1 if i in axes else s for i, s in enumerate(ins[0]) if keep or i not in axes]
+        return [(tuple(out), tys[0])]
+    raise ShapeInferenceError(f"no shape rule for op '{op}' (node '{node.name}')")
+
+
+def infer_shapes(model: ModelProto) -> ModelProto:
+    """Fill ``graph.value_info`` for every intermediate value (in place; returns the model)."""
+    g = model.graph
+    shapes: typing.Dict[str, tuple] = {}
+    types: typing.Dict[str, int] = {}
+    constants = {}
+    for t in g.initializer:
+        shapes[t.name] = tuple(t.dims)
+        types[t.name] = t.data_type
+        constants[t.name] = t.array
+    for v in list(g.input) + list(g.value_info) + list(g.output):
+        if v.shape is not None and all(isinstance(d, int) for d in v.shape):
+            shapes.setdefault(v.name, tuple(v.shape))
+            types.setdefault(v.name, v.elem_type)
+    known_vi = {v.name for v in g.value_info} | {v.name for v in g.output} | {v.name for v in g.input}
+    for node in g.node:
+        results = _infer_node(node, shapes, types, constants)
+        for out_name, (shape, ty) in zip(node.output, results):
+            if out_name in shapes and tuple(shapes[out_name]) != tuple(shape):
+                raise ShapeInferenceError(
+                    f"{node.op_type} '{node.name}': inferred shape {shape} for '{out_name}' "
+                    f"contradicts the declared shape {shapes[out_name]}")
+            shapes[out_name], types[out_name] = tuple(shape), ty
+            if out_name not in known_vi:
+                g.value_info.append(ValueInfoProto(out_name, ty, list(shape)))
+                known_vi.add(out_name)
+    for v in g.output:
+        if v.shape is None and v.name in shapes:
+            v.shape, v.elem_type = list(shapes[v.name]), types[v.name]
+    return model

@@ -109,10 +109,11 @@ int mi355x_conv2d_f32(const float* X, const float* W, const float* bias, float* 
  * The reference has no expansion of its own for this node: the generated class
  * (daceml/onnx/nodes/onnx_op.py:623-640) only has the "onnxruntime"
  * implementation (onnx_op.py:686-687 -> node_codegen.py:321-573).
- * A is [M,K], B is [K,N], Y is [M,N], all C-contiguous; zero points are
- * scalars passed by value. */
+ * A is [M,K], B is [K,N], Y is [M,N], all C-contiguous. The zero points are
+ * the node's optional scalar inputs: DEVICE pointers to one int8 each, read by
+ * the kernel (no host synchronisation); NULL means 0. */
 int mi355x_matmul_integer_i8(const int8_t* A, const int8_t* B,
-                             int32_t a_zero_point, int32_t b_zero_point,
+                             const int8_t* a_zero_point, const int8_t* b_zero_point,
                              int32_t* Y, int64_t M, int64_t N, int64_t K,
                              void* stream);
 

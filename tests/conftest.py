@@ -1,0 +1,51 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def golden():
+    """Committed fixtures: seeded inputs and expectations computed with PyTorch CPU float64
+    (tests/golden/make_golden.py)."""
+    return np.load(os.path.join(GOLDEN_DIR, "hotpath_golden.npz"))
+
+
+@pytest.fixture
+def sdfg_name(request):
+    # same naming rule as the reference's fixture (tests/conftest.py:53-56)
+    return request.node.name.replace("[", "-").replace("]", "").replace("-", "_").replace(".", "_")
+
+
+@pytest.fixture(scope="session")
+def c_oracle():
+    from oracle import c_oracle as c
+    c.build()
+    return c
+
+
+def rel_err(expected, actual):
+    """max |actual - expected| / max |expected|, in float64."""
+    e = np.asarray(expected, dtype=np.float64)
+    a = np.asarray(actual, dtype=np.float64)
+    assert e.shape == a.shape, (e.shape, a.shape)
+    if e.size == 0:
+        return 0.0
+    scale = np.abs(e).max()
+    return float(np.abs(a - e).max() / (scale if scale > 0 else 1.0))
+
+
+#: fp32 parity bar for every floating-point kernel: 1e-4 relative to the largest
+#: magnitude of the expected tensor (integer kernels must be bit-exact)
+FP32_REL_TOL = 1e-4
