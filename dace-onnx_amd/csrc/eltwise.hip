@@ -204,9 +204,15 @@ extern "C" int mi355x_eltwise_f32(int op, const float* A, const float* B, float*
     using namespace mi355x;
     MI355X_REQUIRE(ndim >= 0 && ndim <= MAX_DIMS, "eltwise: ndim %d outside [0, %d]", ndim, MAX_DIMS);
     const bool bin = is_binary(op);
+    MI355X_REQUIRE(ndim == 0 || (shape && a_strides && (!bin || b_strides)), "eltwise: null shape/strides");
+    int64_t total = 1;
+    for (int d = 0; d < ndim; ++d) total *= shape[d] > 0 ? shape[d] : 0;
+    if (total == 0) {
+        for (int d = 0; d < ndim; ++d) MI355X_REQUIRE(shape[d] >= 0, "eltwise: negative extent");
+        return MI355X_OK;
+    }
     MI355X_REQUIRE(A && C, "eltwise: null pointer");
     MI355X_REQUIRE(!bin || B, "eltwise: binary op %d needs B", op);
-    MI355X_REQUIRE(ndim == 0 || (shape && a_strides && (!bin || b_strides)), "eltwise: null shape/strides");
     IndexMap m;
     m.ndim = ndim == 0 ? 1 : ndim;
     for (int d = 0; d < MAX_DIMS; ++d) { m.shape[d] = 1; m.a_strides[d] = 0; m.b_strides[d] = 0; }
@@ -234,7 +240,6 @@ extern "C" int mi355x_permute_b32(const void* X, void* Y, int ndim, const int64_
                                   const int64_t* x_strides, void* stream) {
     using namespace mi355x;
     MI355X_REQUIRE(ndim >= 0 && ndim <= MAX_DIMS, "permute: ndim %d outside [0, %d]", ndim, MAX_DIMS);
-    MI355X_REQUIRE(X && Y, "permute: null pointer");
     MI355X_REQUIRE(ndim == 0 || (shape && x_strides), "permute: null shape/strides");
     IndexMap m;
     m.ndim = ndim == 0 ? 1 : ndim;
@@ -247,6 +252,7 @@ extern "C" int mi355x_permute_b32(const void* X, void* Y, int ndim, const int64_
         n *= shape[d];
     }
     if (n == 0) return MI355X_OK;
+    MI355X_REQUIRE(X && Y, "permute: null pointer");
     collapse(m, false);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t* x = static_cast<const uint32_t*>(X);

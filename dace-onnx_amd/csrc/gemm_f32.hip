@@ -220,7 +220,7 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
                    "gemm: MI355X_EPI_RESIDUAL without residual / r_strides");
     const int64_t batch = batch0 * batch1;
     if (batch == 0 || M == 0 || N == 0) return MI355X_OK;
-    MI355X_REQUIRE(A && B && C, "gemm: null pointer");
+    MI355X_REQUIRE(C && (K == 0 || (A && B)), "gemm: null pointer");
     MI355X_REQUIRE(c_strides[2] >= N || M == 1, "gemm: C row stride %lld < N %lld", (long long)c_strides[2], (long long)N);
 
     GemmArgs p;

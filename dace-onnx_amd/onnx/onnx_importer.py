@@ -88,6 +88,9 @@ class ONNXModel:
         self.do_auto_optimize = auto_optimize
         self.fuse = fuse
         self.use_hip_graph = use_hip_graph
+        for node in model.graph.node:
+            if not has_onnx_node(node.op_type):
+                raise ValueError("Unsupported ONNX operator: '{}'".format(node.op_type))
         if infer_shapes:
             model = _infer_shapes(model)
         graph = model.graph
@@ -169,7 +172,7 @@ class ONNXModel:
                     self.state.add_edge(op_node, conn_name, access, None, memlet)
 
         self._compiled = None
-        self._graph_ready = False
+        self._static_io = None
 
     # -- construction helpers ----------------------------------------------------------
     @staticmethod
@@ -266,11 +269,22 @@ class ONNXModel:
                 v = torch.from_numpy(np.ascontiguousarray(np.asarray(v, dtype=desc.dtype.np_dtype))).to(self.device)
             call[clean_onnx_name(n)] = v
         outputs = collections.OrderedDict()
-        if self.use_hip_graph and getattr(self, "_static_io", None) is not None:
-            s_in, s_out = self._static_io
-            for k, v in call.items():
-                s_in[k].copy_(v)
-            compiled.replay()
+        if self.use_hip_graph:
+            if self._static_io is None:
+                # private input/output buffers: the graph is bound to their addresses
+                s_in = {k: v.clone() for k, v in call.items()}
+                s_out = {}
+                for n in self.outputs:
+                    desc = self.sdfg.arrays[clean_onnx_name(n)]
+                    s_out[clean_onnx_name(n)] = torch.empty(desc.shape, dtype=desc.dtype.as_torch(), device=self.device)
+                compiled(**s_in, **s_out, **self.clean_weights)  # eager run, binds the launch list
+                compiled.capture_graph()
+                self._static_io = (s_in, s_out)
+            else:
+                s_in, s_out = self._static_io
+                for k, v in call.items():
+                    s_in[k].copy_(v)
+                compiled.replay()
             outputs = collections.OrderedDict((n, s_out[clean_onnx_name(n)].clone()) for n in self.outputs)
         else:
             for n in self.outputs:
@@ -278,10 +292,5 @@ class ONNXModel:
                 outputs[n] = torch.empty(desc.shape, dtype=desc.dtype.as_torch(), device=self.device)
             out_kwargs = {clean_onnx_name(n): t for n, t in outputs.items()}
             compiled(**call, **out_kwargs, **self.clean_weights)
-            if self.use_hip_graph:
-                # later calls copy into these buffers and replay one HIP graph
-                compiled.capture_graph()
-                self._static_io = (dict(call), dict(out_kwargs))
-                outputs = collections.OrderedDict((n, t.clone()) for n, t in outputs.items())
         results = [t if use_torch else t.cpu().numpy() for t in outputs.values()]
         return results[0] if len(results) == 1 else tuple(results)

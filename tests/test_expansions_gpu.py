@@ -1,0 +1,313 @@
+"""GPU parity of every "mi355x" expansion against the oracle, through the same
+graph-building code the reference's expansion tests use
+(tests/pure_expansions/test_expansions.py, test_conv_expansion.py,
+tests/test_python_frontend.py): build a one-node SDFG (or use the frontend call
+form), expand, check that the node really became a kernel call, run, compare.
+
+Tolerance: fp32 kernels within 1e-4 of the expected tensor's largest magnitude
+(FP32_REL_TOL); MatMulInteger bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from dace_onnx_amd import sdfg as dace
+import dace_onnx_amd.onnx as donnx
+from dace_onnx_amd.util import utils
+from oracle import pure_ops as O
+from conftest import rel_err, FP32_REL_TOL
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_expanded_to_kernels(sdfg):
+    # the reference asserts a MapEntry exists, i.e. the node did not go to ONNX Runtime
+    assert any(isinstance(n, (dace.KernelCall, dace.AliasNode)) for n, _ in sdfg.all_nodes_recursive())
+    assert not any(isinstance(n, dace.LibraryNode) for n, _ in sdfg.all_nodes_recursive())
+
+
+# ----------------------------------------------------------------------------- MatMul / Gemm
+@pytest.mark.parametrize("a_shape, b_shape", [([2, 4], [4, 3]), ([8, 12, 128, 64], [8, 12, 64, 128]),
+                                              ([8, 128, 768], [768, 3072]), ([3, 5, 7], [7, 2]), ([5, 7], [3, 7, 2]),
+                                              ([2, 1, 33, 65], [3, 65, 17]), ([1, 1], [1, 1]), ([130, 131], [131, 129])])
+def test_matmul_expansion(a_shape, b_shape, sdfg_name):
+    sdfg = dace.SDFG(sdfg_name)
+    rng = np.random.default_rng(0)
+    X = rng.random(a_shape).astype(np.float32)
+    Z = rng.random(b_shape).astype(np.float32)
+    expected_result = O.matmul(X, Z)
+    sdfg.add_array("X", a_shape, dace.float32)
+    sdfg.add_array("Z", b_shape, dace.float32)
+    sdfg.add_array("__return", expected_result.shape, dace.float32)
+    state = sdfg.add_state()
+    access_X = state.add_access("X")
+    access_Z = state.add_access("Z")
+    access_result = state.add_access("__return")
+    op_node = donnx.ONNXMatMul("Matmul")
+    state.add_node(op_node)
+    state.add_edge(access_X, None, op_node, "A", sdfg.make_array_memlet("X"))
+    state.add_edge(access_Z, None, op_node, "B", sdfg.make_array_memlet("Z"))
+    state.add_edge(op_node, "Y", access_result, None, sdfg.make_array_memlet("__return"))
+    sdfg.expand_library_nodes()
+    assert_expanded_to_kernels(sdfg)
+    result = sdfg(X=X, Z=Z)
+    assert np.allclose(expected_result, result)  # the reference's check (test_expansions.py:56)
+    assert rel_err(X.astype(np.float64) @ Z.astype(np.float64), result) < FP32_REL_TOL
+
+
+def test_matmul_python_frontend_form():
+    # tests/test_python_frontend.py:12-22
+    rng = np.random.default_rng(1)
+    A = rng.normal(size=(5, 5)).astype(np.float32)
+    B = rng.normal(size=(5, 3)).astype(np.float32)
+    out = np.zeros((5, 3), np.float32)
+    donnx.ONNXMatMul(A=A.copy(), B=B.copy(), Y=out)
+    assert np.allclose(A @ B, out)
+    with pytest.raises(TypeError, match="Unknown arguments"):
+        donnx.ONNXMatMul(A=A, B=B, Y=out, Q=out)
+
+
+@pytest.mark.parametrize("transA, transB, alpha, c_shape", [(0, 1, 1.0, (9, )), (0, 0, 1.0, None), (1, 0, 0.5, (1, 9)),
+                                                            (1, 1, 2.0, (10, 9)), (0, 1, 1.0, None)])
+def test_gemm(transA, transB, alpha, c_shape):
+    rng = np.random.default_rng(2)
+    M, K, N = 10, 12, 9
+    A = rng.normal(size=(K, M) if transA else (M, K)).astype(np.float32)
+    B = rng.normal(size=(N, K) if transB else (K, N)).astype(np.float32)
+    C = rng.normal(size=c_shape).astype(np.float32) if c_shape else None
+    Y = np.zeros((M, N), np.float32)
+    kwargs = dict(A=A, B=B, Y=Y, transA=transA, transB=transB, alpha=alpha)
+    if C is not None:
+        kwargs["C"] = C
+    donnx.ONNXGemm(**kwargs)
+    assert rel_err(O.gemm(A, B, C, alpha=alpha, transA=transA, transB=transB), Y) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- Conv
+@pytest.mark.parametrize("num_in_channels, kernel_size, num_filters, bias",
+                         [(1, (3, 3), 8, True), (8, (3, 3), 3, False), (8, (5, 5), 3, True), (8, (4, 4), 3, False)])
+def test_conv_simple(num_in_channels, kernel_size, num_filters, bias):
+    # the reference's grid (test_conv_expansion.py:10-64), frontend call form
+    batch_size = 8
+    rng = np.random.default_rng(3)
+    X = rng.random((batch_size, num_in_channels, 32, 32)).astype(np.float32)
+    W = rng.random((num_filters, num_in_channels, *kernel_size)).astype(np.float32)
+    B = rng.random(num_filters).astype(np.float32) if bias else None
+    expected = O.conv2d(X, W, B)
+    dace_Z = np.zeros_like(expected)
+    if bias:
+        donnx.ONNXConv(X=X, W=W, B=B, Y=dace_Z)
+    else:
+        donnx.ONNXConv(X=X, W=W, Y=dace_Z)
+    assert np.allclose(expected, dace_Z, rtol=1e-4, atol=1e-4)
+    assert rel_err(expected, dace_Z) < FP32_REL_TOL
+
+
+def test_conv_config1_stride2():
+    # BASELINE config 1 and the reference's README example (examples/plot_conv.py:43-46)
+    rng = np.random.default_rng(1)
+    X = rng.random((5, 3, 10, 10), dtype=np.float32)
+    W = rng.random((16, 3, 3, 3), dtype=np.float32)
+    Y = np.zeros((5, 16, 4, 4), np.float32)
+    donnx.ONNXConv(X=X, W=W, Y=Y, strides=[2, 2])
+    assert rel_err(O.conv2d(X, W, strides=(2, 2)), Y) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("shape, wshape, attrs", [
+    ((2, 5, 13, 17), (7, 5, 3, 2), dict(pads=[1, 2, 0, 1], strides=[2, 1], dilations=[2, 3])),
+    ((1, 3, 7, 7), (20, 3, 7, 7), dict()),                                     # output 1x1
+    ((3, 4, 9, 9), (65, 4, 1, 1), dict(strides=[3, 3])),                       # 1x1 kernel, odd filter count
+    ((2, 6, 15, 14), (33, 6, 3, 3), dict(auto_pad="SAME_UPPER", strides=[2, 2])),
+    ((1, 2, 30, 31), (4, 2, 5, 3), dict(pads=[2, 1, 2, 1])),                   # OH*OW % 4 != 0: scalar stores
+])
+def test_conv_attributes(shape, wshape, attrs):
+    rng = np.random.default_rng(4)
+    X = rng.normal(size=shape).astype(np.float32)
+    W = rng.normal(size=wshape).astype(np.float32)
+    B = rng.normal(size=wshape[0]).astype(np.float32)
+    strides = tuple(attrs.get("strides", (1, 1)))
+    dil = tuple(attrs.get("dilations", (1, 1)))
+    if attrs.get("auto_pad") == "SAME_UPPER":
+        pads = []
+        for size, s, k in ((shape[2], strides[0], wshape[2]), (shape[3], strides[1], wshape[3])):
+            total = max((-(-size // s) - 1) * s + k - size, 0)
+            pads.append((total // 2, total - total // 2))
+        pads = (pads[0][0], pads[1][0], pads[0][1], pads[1][1])
+    else:
+        pads = tuple(attrs.get("pads", (0, 0, 0, 0)))
+    expected = O.conv2d(X, W, B, strides, pads, dil)
+    Y = np.zeros_like(expected)
+    donnx.ONNXConv(X=X, W=W, B=B, Y=Y, **attrs)
+    assert rel_err(expected, Y) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- Softmax / LayerNorm
+@pytest.mark.parametrize("axis", [0, -1])
+def test_softmax(axis, sdfg_name):
+    # tests/pure_expansions/test_expansions.py:345-379
+    X = np.random.default_rng(5).normal(scale=10, size=(2, 4, 10)).astype(np.float32)
+    torch_result = torch.nn.functional.softmax(torch.Tensor(X), dim=axis).numpy()
+    sdfg = dace.SDFG(sdfg_name)
+    sdfg.add_array("X", [2, 4, 10], dace.float32)
+    sdfg.add_array("__return", torch_result.shape, dace.float32)
+    state = sdfg.add_state()
+    access_X = state.add_access("X")
+    access_result = state.add_access("__return")
+    op_node = donnx.ONNXSoftmax("softmax")
+    op_node.axis = axis
+    state.add_node(op_node)
+    state.add_edge(access_X, None, op_node, "input", sdfg.make_array_memlet("X"))
+    state.add_edge(op_node, "output", access_result, None, sdfg.make_array_memlet("__return"))
+    sdfg.expand_library_nodes()
+    assert_expanded_to_kernels(sdfg)
+    result = sdfg(X=X)
+    assert np.linalg.norm(torch_result - result) < 1e-5
+    assert rel_err(O.softmax(X, axis=axis), result) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("shape", [(8, 12, 16, 128), (7, 64), (33, 256), (5, 1000), (3, 2048), (2, 5000), (4, 36),
+                                   (3, 1), (5, 7), (2, 130)])
+def test_softmax_row_lengths(shape):
+    X = np.random.default_rng(6).normal(scale=4, size=shape).astype(np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXSoftmax(input=X, output=Y, axis=-1)
+    assert rel_err(O.softmax(X), Y) < FP32_REL_TOL
+    assert np.allclose(Y.sum(-1), 1.0, atol=1e-5)
+
+
+def test_softmax_large_values_and_middle_axis():
+    X = np.array([[1000.0, 999.0, -1000.0, 0.0]] * 3, np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXSoftmax(input=X, output=Y, axis=1)
+    assert np.isfinite(Y).all() and rel_err(O.softmax(X), Y) < FP32_REL_TOL
+    X = np.random.default_rng(7).normal(size=(3, 17, 5, 9)).astype(np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXSoftmax(input=X, output=Y, axis=1)
+    assert rel_err(O.softmax(X, axis=1), Y) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("shape, axis", [((8, 16, 768), -1), ((5, 256), -1), ((3, 1000), 1), ((2, 4096), -1),
+                                         ((2, 5000), -1), ((3, 30), -1), ((4, 6, 48), 1), ((3, 1), -1)])
+def test_layer_normalization(shape, axis):
+    rng = np.random.default_rng(8)
+    X = rng.normal(size=shape).astype(np.float32)
+    norm_shape = shape[axis % len(shape):]
+    g = rng.normal(1.0, 0.02, size=norm_shape).astype(np.float32)
+    b = rng.normal(0.0, 0.02, size=norm_shape).astype(np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXLayerNormalization(X=X, Scale=g, B=b, Y=Y, axis=axis, epsilon=1e-12)
+    assert rel_err(O.layer_normalization(X, g, b, axis=axis, epsilon=1e-12), Y) < FP32_REL_TOL
+    Y2 = np.zeros_like(X)
+    donnx.ONNXLayerNormalization(X=X, Scale=g, Y=Y2, axis=axis)  # no bias, default epsilon
+    assert rel_err(O.layer_normalization(X, g, None, axis=axis, epsilon=1e-5), Y2) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- elementwise
+@pytest.mark.parametrize("a_shape, b_shape", [((8, 16, 768), (768, )), ((8, 16, 768), (8, 16, 768)), ((5, 1, 7), (3, 1)),
+                                              ((4, 6), ()), ((1, ), (2, 3, 4)), ((768, ), (2, 4, 768)), ((3, 5), (3, 1))])
+@pytest.mark.parametrize("op", ["Add", "Sub", "Mul", "Div"])
+def test_binary_broadcast(op, a_shape, b_shape):
+    rng = np.random.default_rng(9)
+    A = rng.normal(size=a_shape).astype(np.float32)
+    B = (rng.random(size=b_shape) + 0.5).astype(np.float32)
+    expected = getattr(O, op.lower())(A, B)
+    C = np.zeros(expected.shape, np.float32)
+    getattr(donnx, "ONNX" + op)(A=A, B=B, C=C)
+    assert np.array_equal(expected, C) or rel_err(expected, C) < 1e-6
+
+
+@pytest.mark.parametrize("shape", [(8, 16, 3072), (7, ), (1, 3, 5), (4097, )])
+def test_unary_ops(shape):
+    X = np.random.default_rng(10).normal(scale=2, size=shape).astype(np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXRelu(X=X, Y=Y)
+    assert np.array_equal(O.relu(X), Y)
+    donnx.ONNXGelu(X=X, Y=Y)
+    assert rel_err(O.gelu(X), Y) < FP32_REL_TOL
+    donnx.ONNXErf(input=X, output=Y)
+    assert rel_err(O.erf(X), Y) < FP32_REL_TOL
+    donnx.ONNXSqrt(X=np.abs(X), Y=Y)
+    assert rel_err(O.sqrt(np.abs(X)), Y) < 1e-6
+
+
+# ----------------------------------------------------------------------------- data movement
+@pytest.mark.parametrize("shape, perm", [((8, 16, 12, 64), (0, 2, 1, 3)), ((2, 12, 16, 64), (0, 1, 3, 2)),
+                                         ((5, 7), None), ((3, 4, 5), (2, 0, 1)), ((70, 130), (1, 0)), ((6, ), (0, ))])
+def test_transpose(shape, perm):
+    X = np.random.default_rng(11).normal(size=shape).astype(np.float32)
+    expected = O.transpose(X, perm)
+    Y = np.zeros(expected.shape, np.float32)
+    kwargs = {} if perm is None else {"perm": list(perm)}
+    donnx.ONNXTranspose(data=X, transposed=Y, **kwargs)
+    assert np.array_equal(expected, Y)
+
+
+def test_reshape_is_a_view_inside_a_graph():
+    # Reshape between two kernels moves no data: the SDFG has two kernel calls and one alias
+    sdfg = dace.SDFG("reshape_chain")
+    sdfg.add_array("X", [4, 6], dace.float32)
+    sdfg.add_array("shape", [3], dace.int64)
+    sdfg.add_transient("r", [4, 6], dace.float32)
+    sdfg.add_transient("v", [2, 3, 4], dace.float32)
+    sdfg.add_array("__return", [2, 3, 4], dace.float32)
+    st = sdfg.add_state()
+    relu, resh, gelu = donnx.ONNXRelu("relu"), donnx.ONNXReshape("reshape"), donnx.ONNXGelu("gelu")
+    ar, av = st.add_access("r"), st.add_access("v")
+    st.add_edge(st.add_read("X"), None, relu, "X", sdfg.make_array_memlet("X"))
+    st.add_edge(relu, "Y", ar, None, sdfg.make_array_memlet("r"))
+    st.add_edge(ar, None, resh, "data", sdfg.make_array_memlet("r"))
+    st.add_edge(st.add_read("shape"), None, resh, "shape", sdfg.make_array_memlet("shape"))
+    st.add_edge(resh, "reshaped", av, None, sdfg.make_array_memlet("v"))
+    st.add_edge(av, None, gelu, "X", sdfg.make_array_memlet("v"))
+    st.add_edge(gelu, "Y", st.add_write("__return"), None, sdfg.make_array_memlet("__return"))
+    utils.expand_onnx_nodes(sdfg)
+    kinds = [type(n).__name__ for n, _ in sdfg.all_nodes_recursive() if isinstance(n, (dace.KernelCall, dace.AliasNode))]
+    assert sorted(kinds) == ["AliasNode", "KernelCall", "KernelCall"]
+    X = np.random.default_rng(12).normal(size=(4, 6)).astype(np.float32)
+    out = sdfg(X=X, shape=np.array([2, 3, 4], np.int64))
+    assert rel_err(O.gelu(O.relu(X)).reshape(2, 3, 4), out) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- MatMulInteger
+@pytest.mark.parametrize("M, N, K, za, zb", [(128, 128, 64, 0, 0), (128, 128, 64, 3, -2), (512, 384, 768, 3, -2),
+                                             (100, 52, 37, 5, 7), (130, 260, 48, -128, 127), (1, 1, 1, 1, 1),
+                                             (33, 2, 16, 0, 9), (7, 129, 1000, -7, 0)])
+def test_matmul_integer_bit_exact(M, N, K, za, zb):
+    rng = np.random.default_rng(13)
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    Y = np.zeros((M, N), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array(za, np.int8), b_zero_point=np.array(zb, np.int8), Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B, za, zb), Y)
+
+
+def test_matmul_integer_without_zero_points_and_extremes():
+    A = np.full((64, 768), -128, np.int8)
+    B = np.full((768, 32), -128, np.int8)
+    Y = np.zeros((64, 32), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, Y=Y)
+    assert np.all(Y == 768 * 128 * 128)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array([127], np.int8), b_zero_point=np.array([127], np.int8), Y=Y)
+    assert np.all(Y == 768 * 255 * 255)
+
+
+# ----------------------------------------------------------------------------- edge cases
+def test_empty_inputs():
+    X = np.zeros((0, 128), np.float32)
+    Y = np.zeros((0, 128), np.float32)
+    donnx.ONNXSoftmax(input=X, output=Y, axis=-1)
+    donnx.ONNXRelu(X=X, Y=Y)
+    A, B, C = np.zeros((0, 8), np.float32), np.zeros((8, 4), np.float32), np.zeros((0, 4), np.float32)
+    donnx.ONNXMatMul(A=A, B=B, Y=C)
+    # K == 0: the product is all zeros
+    A, B, C = np.zeros((3, 0), np.float32), np.zeros((0, 4), np.float32), np.ones((3, 4), np.float32)
+    donnx.ONNXMatMul(A=A, B=B, Y=C)
+    assert np.all(C == 0)
+
+
+def test_torch_tensors_stay_on_device():
+    x = torch.randn(64, 128, device="cuda")
+    y = torch.empty_like(x)
+    donnx.ONNXSoftmax(input=x, output=y, axis=-1)
+    torch.cuda.synchronize()
+    assert rel_err(O.softmax(x.cpu().numpy()), y.cpu().numpy()) < FP32_REL_TOL

@@ -1,0 +1,274 @@
+"""Pins the oracle (CPU restatement of the reference's expansions).
+
+The reference's tests hold no golden vectors: each recomputes its expectation
+with numpy / PyTorch (tests/pure_expansions/test_expansions.py:29,349;
+test_conv_expansion.py:30-35). The same comparators are used here, plus the
+committed fixtures (PyTorch float64), closed forms, invariants and brute force,
+chosen so that a dropped term, a wrong sign/index or a transposed operand fails.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import pure_ops as O
+from conftest import rel_err
+
+TOL = 2e-6  # oracle is fp32 numpy; comparators are float64
+
+
+# ----------------------------------------------------------------------------- golden fixtures
+def test_golden_conv_config1(golden):
+    y = O.conv2d(golden["conv1_X"], golden["conv1_W"], strides=(2, 2))
+    assert y.shape == (5, 16, 4, 4)
+    assert rel_err(golden["conv1_Y"], y) < TOL
+
+
+def test_golden_conv_pads_dilation_bias_relu(golden):
+    y = O.relu(O.conv2d(golden["conv2_X"], golden["conv2_W"], golden["conv2_B"], strides=(2, 1),
+                        pads=(1, 2, 0, 1), dilations=(1, 2)))
+    assert rel_err(golden["conv2_Y"], y) < TOL
+
+
+def test_golden_softmax_layernorm_gelu(golden):
+    assert rel_err(golden["softmax_Y"], O.softmax(golden["softmax_X"], axis=-1)) < TOL
+    assert rel_err(golden["ln_Y"], O.layer_normalization(golden["ln_X"], golden["ln_gamma"], golden["ln_beta"],
+                                                         axis=-1, epsilon=1e-12)) < TOL
+    assert rel_err(golden["gelu_Y"], O.gelu(golden["gelu_X"])) < TOL
+
+
+def test_golden_matmul_gemm(golden):
+    assert rel_err(golden["matmul_Y"], O.matmul(golden["matmul_A"], golden["matmul_B"])) < TOL
+    assert rel_err(golden["gemm_Y"], O.gemm(golden["gemm_A"], golden["gemm_B"], golden["gemm_C"], transB=1)) < TOL
+
+
+def test_golden_matmul_integer(golden):
+    y = O.matmul_integer(golden["mmi_A"], golden["mmi_B"], 3, -2)
+    assert y.dtype == np.int32 and np.array_equal(y, golden["mmi_Y"])
+
+
+def test_golden_bert_layer(golden):
+    hidden, heads, ffn, bsz, seq = (int(v) for v in golden["bert_meta"])
+    w = {k[len("bert_"):]: golden[k] for k in golden.files if k.startswith("bert_") and k not in
+         ("bert_x", "bert_y", "bert_meta")}
+    y = O.bert_layer(golden["bert_x"], w, heads=heads)
+    assert y.shape == (bsz, seq, hidden)
+    assert rel_err(golden["bert_y"], y) < 5e-6
+
+
+# ----------------------------------------------------------------------------- matmul / gemm
+def test_matmul_einsum_strings():
+    # the strings PureMatMul produces (pure_implementations.py:151-210)
+    assert O.matmul_einsum_string(2, 2) == "ik,kj->ij"
+    assert O.matmul_einsum_string(3, 2) == "aik,kj->aij"
+    assert O.matmul_einsum_string(4, 4) == "baik,bakj->baij"
+    assert O.matmul_einsum_string(2, 3) == "ik,akj->aij"
+    with pytest.raises(ValueError):
+        O.matmul_einsum_string(1, 2)
+
+
+@pytest.mark.parametrize("a_shape, b_shape", [([2, 4], [4, 3]), ([8, 12, 16, 8], [8, 12, 8, 16]),
+                                              ([3, 5, 7], [7, 2]), ([5, 7], [3, 7, 2]), ([2, 1, 4, 6], [3, 6, 5])])
+def test_matmul_vs_numpy_float64(a_shape, b_shape):
+    rng = np.random.default_rng(0)
+    A = rng.random(a_shape).astype(np.float32)
+    B = rng.random(b_shape).astype(np.float32)
+    assert rel_err(A.astype(np.float64) @ B.astype(np.float64), O.matmul(A, B)) < TOL
+
+
+def test_matmul_bruteforce_small():
+    rng = np.random.default_rng(1)
+    A = rng.normal(size=(5, 7)).astype(np.float32)
+    B = rng.normal(size=(7, 6)).astype(np.float32)
+    ref = np.zeros((5, 6))
+    for i in range(5):
+        for j in range(6):
+            for k in range(7):
+                ref[i, j] += float(A[i, k]) * float(B[k, j])
+    assert rel_err(ref, O.matmul(A, B)) < TOL
+    # a transposed operand must fail this check
+    assert rel_err(ref, O.matmul(A, np.ascontiguousarray(B.T).reshape(7, 6))) > 1e-2
+
+
+def test_gemm_attributes():
+    rng = np.random.default_rng(2)
+    A = rng.normal(size=(6, 4)).astype(np.float32)
+    B = rng.normal(size=(6, 5)).astype(np.float32)
+    C = rng.normal(size=(4, 5)).astype(np.float32)
+    ref = 0.5 * (A.astype(np.float64).T @ B.astype(np.float64)) + 2.0 * C
+    assert rel_err(ref, O.gemm(A, B, C, alpha=0.5, beta=2.0, transA=1, transB=0)) < TOL
+
+
+# ----------------------------------------------------------------------------- conv
+@pytest.mark.parametrize("num_in_channels, kernel_size, num_filters, bias",
+                         [(1, (3, 3), 8, True), (8, (3, 3), 3, False), (8, (5, 5), 3, True), (8, (4, 4), 3, False)])
+def test_conv_reference_test_grid(num_in_channels, kernel_size, num_filters, bias):
+    # the parameter grid of the reference's test_conv_simple (test_conv_expansion.py:10-13)
+    rng = np.random.default_rng(3)
+    X = rng.random((8, num_in_channels, 32, 32)).astype(np.float32)
+    W = rng.random((num_filters, num_in_channels, *kernel_size)).astype(np.float32)
+    B = rng.random(num_filters).astype(np.float32) if bias else None
+    ref = F.conv2d(torch.from_numpy(X).double(), torch.from_numpy(W).double(),
+                   bias=None if B is None else torch.from_numpy(B).double()).numpy()
+    assert rel_err(ref, O.conv2d(X, W, B)) < TOL
+
+
+@pytest.mark.parametrize("strides, pads, dil", [((2, 2), (0, 0, 0, 0), (1, 1)), ((1, 1), (1, 1, 1, 1), (1, 1)),
+                                                ((2, 3), (2, 0, 1, 3), (1, 1)), ((1, 2), (1, 2, 2, 1), (2, 3))])
+def test_conv_stride_pad_dilation_vs_torch_and_bruteforce(strides, pads, dil):
+    rng = np.random.default_rng(4)
+    X = rng.normal(size=(2, 3, 11, 13)).astype(np.float32)
+    W = rng.normal(size=(4, 3, 3, 2)).astype(np.float32)
+    B = rng.normal(size=4).astype(np.float32)
+    xp = F.pad(torch.from_numpy(X).double(), (pads[1], pads[3], pads[0], pads[2]))
+    ref = F.conv2d(xp, torch.from_numpy(W).double(), torch.from_numpy(B).double(), stride=strides,
+                   dilation=dil).numpy()
+    y = O.conv2d(X, W, B, strides, pads, dil)
+    assert y.shape == ref.shape == O.conv_output_shape(X.shape, W.shape, strides, pads, dil)
+    assert rel_err(ref, y) < TOL
+    assert rel_err(ref, O.conv2d_bruteforce(X, W, B, strides, pads, dil)) < 1e-12 + TOL
+
+
+def test_conv_stride_is_not_ignored():
+    # PureConv2D drops the stride (img_op_implementations.py:278); the parity target keeps it
+    rng = np.random.default_rng(5)
+    X = rng.random((1, 1, 8, 8)).astype(np.float32)
+    W = rng.random((1, 1, 3, 3)).astype(np.float32)
+    full = O.conv2d(X, W)
+    strided = O.conv2d(X, W, strides=(2, 2))
+    assert strided.shape == (1, 1, 3, 3)
+    assert np.allclose(strided, full[:, :, ::2, ::2])
+
+
+# ----------------------------------------------------------------------------- softmax / layernorm / gelu
+@pytest.mark.parametrize("axis", [0, 1, -1])
+def test_softmax_vs_torch(axis):
+    rng = np.random.default_rng(6)
+    X = rng.normal(scale=10, size=(2, 4, 10)).astype(np.float32)  # the reference's case (test_expansions.py:347)
+    ref = F.softmax(torch.from_numpy(X).double(), dim=axis).numpy()
+    y = O.softmax(X, axis=axis)
+    assert np.linalg.norm(ref - y) < 1e-5  # the reference's own bar (test_expansions.py:379)
+    assert rel_err(ref, y) < TOL
+
+
+def test_softmax_invariants():
+    rng = np.random.default_rng(7)
+    X = rng.normal(size=(6, 128)).astype(np.float32)
+    y = O.softmax(X)
+    assert np.allclose(y.sum(-1), 1.0, atol=1e-6)
+    assert np.allclose(O.softmax(X + 3.0), y, atol=1e-6)          # shift invariance
+    assert np.allclose(O.softmax(np.full((2, 5), 4.0, np.float32)), 0.2)  # constant row -> 1/n
+    big = np.array([[1000.0, 0.0]], np.float32)                    # max subtraction keeps it finite
+    assert np.allclose(O.softmax(big), [[1.0, 0.0]])
+
+
+def test_layernorm_vs_torch_and_special_cases():
+    rng = np.random.default_rng(8)
+    X = rng.normal(size=(4, 9, 48)).astype(np.float32)
+    g = rng.normal(1, 0.1, size=48).astype(np.float32)
+    b = rng.normal(0, 0.1, size=48).astype(np.float32)
+    ref = F.layer_norm(torch.from_numpy(X).double(), (48, ), torch.from_numpy(g).double(),
+                       torch.from_numpy(b).double(), eps=1e-12).numpy()
+    assert rel_err(ref, O.layer_normalization(X, g, b, epsilon=1e-12)) < TOL
+    # two trailing axes
+    g2 = rng.normal(1, 0.1, size=(9, 48)).astype(np.float32)
+    ref2 = F.layer_norm(torch.from_numpy(X).double(), (9, 48), torch.from_numpy(g2).double(), None, eps=1e-5).numpy()
+    assert rel_err(ref2, O.layer_normalization(X, g2, None, axis=1, epsilon=1e-5)) < TOL
+    # gamma = 1, beta = 0 -> zero mean, unit (biased) variance
+    y = O.layer_normalization(X, np.ones(48, np.float32), np.zeros(48, np.float32), epsilon=1e-12)
+    assert np.allclose(y.mean(-1), 0, atol=1e-6) and np.allclose(y.var(-1), 1, atol=1e-4)
+    # constant row -> beta
+    c = O.layer_normalization(np.full((1, 48), 7.0, np.float32), g, b, epsilon=1e-5)
+    assert np.allclose(c, b, atol=1e-6)
+
+
+def test_gelu_erf_relu_closed_forms():
+    x = np.linspace(-6, 6, 101).astype(np.float32)
+    ref = np.array([0.5 * v * (1 + math.erf(v / math.sqrt(2))) for v in x.astype(np.float64)])
+    assert rel_err(ref, O.gelu(x)) < TOL
+    assert rel_err(F.gelu(torch.from_numpy(x).double()).numpy(), O.gelu(x)) < TOL
+    assert rel_err(np.array([math.erf(v) for v in x.astype(np.float64)]), O.erf(x)) < TOL
+    assert np.array_equal(O.relu(x), np.where(x > 0, x, 0).astype(np.float32))
+    assert O.relu(x).dtype == np.float32
+
+
+def test_add_broadcasting():
+    rng = np.random.default_rng(9)
+    a = rng.normal(size=(8, 16, 24)).astype(np.float32)
+    b = rng.normal(size=(24, )).astype(np.float32)
+    assert np.array_equal(O.add(a, b), a + b[None, None, :])
+    assert O.add(a, a).shape == a.shape
+
+
+# ----------------------------------------------------------------------------- matmul integer
+def test_matmul_integer_identity_and_extremes():
+    rng = np.random.default_rng(10)
+    A = rng.integers(-128, 128, size=(33, 70), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(70, 21), dtype=np.int8)
+    za, zb = 3, -2
+    y = O.matmul_integer(A, B, za, zb)
+    a64, b64 = A.astype(np.int64), B.astype(np.int64)
+    ident = a64 @ b64 - zb * a64.sum(1, keepdims=True) - za * b64.sum(0, keepdims=True) + 70 * za * zb
+    assert np.array_equal(y, ident.astype(np.int32))
+    # brute force on one row
+    row = [sum((int(A[0, k]) - za) * (int(B[k, j]) - zb) for k in range(70)) for j in range(21)]
+    assert np.array_equal(y[0], np.array(row, dtype=np.int32))
+    # extreme values: (-128 - 127) * (-128 - 127) * K
+    Ae = np.full((2, 768), -128, np.int8)
+    Be = np.full((768, 2), -128, np.int8)
+    assert np.all(O.matmul_integer(Ae, Be, 127, 127) == 768 * 255 * 255)
+    # swapping the zero points must change the result
+    assert not np.array_equal(y, O.matmul_integer(A, B, zb, za))
+
+
+# ----------------------------------------------------------------------------- C restatement vs numpy restatement
+def test_c_oracle_matches_numpy_oracle(c_oracle):
+    rng = np.random.default_rng(11)
+    X = rng.normal(size=(3, 5, 12, 10)).astype(np.float32)
+    W = rng.normal(size=(6, 5, 3, 3)).astype(np.float32)
+    B = rng.normal(size=6).astype(np.float32)
+    for strides, pads, dil in (((1, 1), (1, 1, 1, 1), (1, 1)), ((2, 2), (0, 0, 0, 0), (1, 1)), ((2, 1), (1, 0, 2, 1), (1, 2))):
+        assert rel_err(O.conv2d(X, W, B, strides, pads, dil), c_oracle.conv2d(X, W, B, strides, pads, dil)) < 1e-5
+    x = rng.normal(size=(7, 128)).astype(np.float32)
+    assert rel_err(O.softmax(x), c_oracle.softmax(x)) < 1e-6
+    g = rng.normal(1, 0.02, size=128).astype(np.float32)
+    b = rng.normal(0, 0.02, size=128).astype(np.float32)
+    assert rel_err(O.layer_normalization(x, g, b, epsilon=1e-12), c_oracle.layer_normalization(x, g, b, 1e-12)) < 1e-5
+    assert rel_err(O.gelu(x), c_oracle.gelu(x)) < 1e-6
+    A = rng.integers(-128, 128, size=(17, 40), dtype=np.int8)
+    Bm = rng.integers(-128, 128, size=(40, 23), dtype=np.int8)
+    assert np.array_equal(O.matmul_integer(A, Bm, 3, -2), c_oracle.matmul_integer(A, Bm, 3, -2))
+    a = rng.normal(size=(9, 14)).astype(np.float32)
+    bb = rng.normal(size=(14, 11)).astype(np.float32)
+    assert rel_err(O.matmul(a, bb), c_oracle.matmul(a, bb)) < 1e-5
+
+
+def test_bert_layer_against_transformers():
+    """The composition is the module the reference tests (BertLayer, test_bert_encoder.py:17)."""
+    from transformers import BertConfig
+    from transformers.models.bert.modeling_bert import BertLayer
+    hidden, heads, ffn, bsz, seq = 64, 4, 128, 2, 12
+    cfg = BertConfig(hidden_size=hidden, num_attention_heads=heads, intermediate_size=ffn, hidden_act="gelu",
+                     layer_norm_eps=1e-12, attention_probs_dropout_prob=0.0, hidden_dropout_prob=0.0)
+    cfg._attn_implementation = "eager"
+    layer = BertLayer(cfg).eval()
+    rng = np.random.default_rng(12)
+    w = O.bert_layer_weights(rng, hidden=hidden, ffn=ffn)
+    for k in ("bq", "bk", "bv", "bo", "b1", "b2"):
+        w[k] = rng.normal(0, 0.02, size=w[k].shape).astype(np.float32)
+    x = rng.normal(size=(bsz, seq, hidden)).astype(np.float32)
+    t = torch.from_numpy
+    with torch.no_grad():
+        att, so = layer.attention.self, layer.attention.output
+        for lin, wn, bn in ((att.query, "wq", "bq"), (att.key, "wk", "bk"), (att.value, "wv", "bv"),
+                            (so.dense, "wo", "bo"), (layer.intermediate.dense, "w1", "b1"),
+                            (layer.output.dense, "w2", "b2")):
+            lin.weight.copy_(t(w[wn]).T)
+            lin.bias.copy_(t(w[bn]))
+        so.LayerNorm.weight.copy_(t(w["ln1_g"])); so.LayerNorm.bias.copy_(t(w["ln1_b"]))
+        layer.output.LayerNorm.weight.copy_(t(w["ln2_g"])); layer.output.LayerNorm.bias.copy_(t(w["ln2_b"]))
+        ref = layer(t(x))
+        ref = (ref[0] if isinstance(ref, (tuple, list)) else ref).numpy()
+    assert rel_err(ref, O.bert_layer(x, w, heads=heads)) < 5e-6
