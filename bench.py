@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the ONNX library-node hot path on one MI355X.
+
+A step is one BERT-base encoder layer (B=8, S=128, hidden 768, 12 heads, FFN
+3072, fp32) run through ``ONNXModel`` with the "mi355x" expansions: the
+configuration the headline metric is quoted on. Inputs and weights are
+synthetic (seeded) and resident in HBM before the timed region. The launch
+sequence is replayed as one HIP graph per step.
+
+Prints one JSON line:
+  value / ms_per_step   milliseconds per encoder layer (lower is better)
+  roofline              the dominant kernel (the fp32 MFMA GEMM): algorithmic FLOP
+                        of all GEMM launches of a layer / their measured durations
+  cpu_baseline          the CPU restatement of the reference's expansion of the
+                        same layer (oracle), timed on the host cores of this box
+  kernels               per-kernel roofline rows (every launch of the layer, plus
+                        the stand-alone Softmax / LayerNorm / Conv / MatMulInteger
+                        configurations), each measured live with HIP events
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# published MI355X peaks (dense)
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_INT8_MFMA_TOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+
+def graph_time_us(launch, reps=50, replays=5):
+    """Average duration of one launch: `reps` back-to-back launches recorded in a
+    HIP graph (no host launch gaps), replayed between two HIP events on the
+    stream the kernels run on."""
+    import torch
+    launch()  # warm-up, loads the code object
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(reps):
+            launch()
+    g.replay()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(replays):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) * 1e3 / reps)
+    return best
+
+
+def algorithmic_work(name, args):
+    """(flops, bytes) of one launch from its C-ABI arguments (fp32 unless stated)."""
+    if name == "mi355x_gemm_f32":
+        b0, b1, M, N, K = args[5:10]
+        epi = args[15]
+        flops = 2.0 * b0 * b1 * M * N * K
+        nbytes = 4.0 * b0 * b1 * (M * K + K * N + M * N * (2 if epi & 8 else 1))
+        return flops, nbytes
+    if name == "mi355x_softmax_f32":
+        outer, n, inner = args[2:5]
+        return 0.0, 8.0 * outer * n * inner
+    if name == "mi355x_layernorm_f32":
+        rows, cols = args[4:6]
+        return 0.0, 8.0 * rows * cols + 8.0 * cols
+    if name == "mi355x_eltwise_f32":
+        shape = args[5]
+        n = 1
+        for v in shape:
+            n *= v
+        reads = 2 if args[0] < 16 else 1
+        return 0.0, 4.0 * n * (reads + 1)
+    if name == "mi355x_permute_b32":
+        n = 1
+        for v in args[3]:
+            n *= v
+        return 0.0, 8.0 * n
+    return 0.0, 0.0
+
+
+def kernel_row(label, us, flops=0.0, nbytes=0.0, bound=None, peak=None):
+    row = {"kernel": label, "us": round(us, 3)}
+    if flops:
+        row["tflops"] = round(flops / us / 1e6, 2)
+    if nbytes:
+        row["gbs"] = round(nbytes / us / 1e3, 1)
+    if bound == "mfma":
+        row.update(bound="mfma", frac=round(flops / us / 1e6 / (peak or PEAK_FP32_MFMA_TFLOPS), 4))
+    elif bound == "hbm":
+        row.update(bound="hbm", frac=round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4))
+    return row
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline rows")
+    ap.add_argument("--eager", action="store_true", help="time host-issued launches instead of HIP-graph replay")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this path has no multi-GPU part (got --gpus {args.gpus}); "
+              f"run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import dace_onnx_amd.onnx as donnx
+    from dace_onnx_amd import _lib
+    from dace_onnx_amd.testing.graphs import bert_encoder_layer_model
+    from oracle import pure_ops  # checker / CPU baseline only
+
+    if not torch.cuda.is_available():
+        print("bench.py needs the MI355X (no HIP device visible)", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.library()
+    torch.cuda.set_device(0)
+
+    # ---- workload: BASELINE config 3 -------------------------------------------------
+    B, S, H, HEADS, FFN = 8, 128, 768, 12, 3072
+    rng = np.random.default_rng(3)
+    weights = pure_ops.bert_layer_weights(rng, hidden=H, ffn=FFN)
+    x_host = rng.normal(size=(B, S, H)).astype(np.float32)
+    model = donnx.ONNXModel("bert_base_encoder_layer", bert_encoder_layer_model(weights, B, S, HEADS))
+    x = torch.from_numpy(x_host).cuda()
+    y = model(x)  # compiles, binds
+    compiled = model.compile_and_init()
+    # parity gate inside the benchmark: a fast wrong layer is not a result
+    expected = pure_ops.bert_layer(x_host, weights, heads=HEADS)
+    err = float(np.abs(y.cpu().numpy().astype(np.float64) - expected).max() / np.abs(expected).max())
+    if not err < 1e-4:
+        print(f"parity check failed: max rel err {err:.3e}", file=sys.stderr)
+        sys.exit(1)
+
+    out = torch.empty_like(y)
+    call_kwargs = {"x": x, "y": out, **model.clean_weights}
+    compiled(**call_kwargs)
+    if args.eager:
+        def step():
+            compiled(**call_kwargs)
+    else:
+        compiled.capture_graph()
+        step = compiled.replay
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    torch.cuda.synchronize()
+    final_err = float(np.abs(out.cpu().numpy().astype(np.float64) - expected).max() / np.abs(expected).max())
+    assert final_err < 1e-4, final_err
+
+    # ---- per-kernel durations, HIP events on the launch stream -----------------------------
+    kernels = []
+    gemm_flops = gemm_us = 0.0
+    if not args.no_kernels:
+        for node, relaunch in compiled.bound_launches():
+            name = node.function
+            plain = [a.values if hasattr(a, "values") else a for a in node.args]
+            flops, nbytes = algorithmic_work(name, plain)
+            us = graph_time_us(relaunch)
+            if name == "mi355x_gemm_f32":
+                gemm_flops += flops
+                gemm_us += us
+                label = "gemm_f32 b{}x{} {}x{}x{} epi={}".format(*plain[5:10], plain[15])
+                kernels.append(kernel_row(label, us, flops, nbytes, "mfma"))
+            else:
+                label = name.replace("mi355x_", "") + " " + "x".join(str(v) for v in (plain[5] if name == "mi355x_eltwise_f32"
+                                                                                     else plain[3] if name == "mi355x_permute_b32"
+                                                                                     else plain[2:5] if name == "mi355x_softmax_f32"
+                                                                                     else plain[4:6]))
+                kernels.append(kernel_row(label, us, 0.0, nbytes, "hbm"))
+
+        # stand-alone configurations of the metric (BASELINE configs 2, 4, 5)
+        st = _lib.current_stream
+        xs = torch.randn(12288, 128, device="cuda")
+        ys = torch.empty_like(xs)
+        us = graph_time_us(lambda: lib.mi355x_softmax_f32(xs.data_ptr(), ys.data_ptr(), 12288, 128, 1, st()))
+        kernels.append(kernel_row("cfg2 softmax 8x12x128x128", us, 0.0, 12582912.0, "hbm"))
+        xl = torch.randn(1024, 768, device="cuda")
+        yl = torch.empty_like(xl)
+        g_, b_ = torch.randn(768, device="cuda"), torch.randn(768, device="cuda")
+        us = graph_time_us(lambda: lib.mi355x_layernorm_f32(xl.data_ptr(), g_.data_ptr(), b_.data_ptr(), yl.data_ptr(),
+                                                            1024, 768, 1e-12, st()))
+        kernels.append(kernel_row("cfg2 layernorm 8x128x768", us, 0.0, 6297600.0, "hbm"))
+        xc = torch.randn(32, 64, 56, 56, device="cuda")
+        wc = torch.randn(64, 64, 3, 3, device="cuda") * (2.0 / 576) ** 0.5
+        bc = torch.zeros(64, device="cuda")
+        yc = torch.empty(32, 64, 56, 56, device="cuda")
+        pads, ones = _lib.i64_array([1, 1, 1, 1]), _lib.i64_array([1, 1])
+        us = graph_time_us(lambda: lib.mi355x_conv2d_f32(xc.data_ptr(), wc.data_ptr(), bc.data_ptr(), yc.data_ptr(), 32, 64,
+                                                         56, 56, 64, 3, 3, pads, ones, ones, 3, st()), reps=20)
+        kernels.append(kernel_row("cfg4 conv+relu 32x64x56x56 k3 p1", us, 7398752256.0, 51527680.0, "mfma"))
+        ai = torch.randint(-128, 128, (4096, 768), dtype=torch.int8, device="cuda")
+        bi = torch.randint(-128, 128, (768, 3072), dtype=torch.int8, device="cuda")
+        za, zb = torch.tensor([3], dtype=torch.int8, device="cuda"), torch.tensor([-2], dtype=torch.int8, device="cuda")
+        yi = torch.empty(4096, 3072, dtype=torch.int32, device="cuda")
+        us = graph_time_us(lambda: lib.mi355x_matmul_integer_i8(ai.data_ptr(), bi.data_ptr(), za.data_ptr(), zb.data_ptr(),
+                                                                yi.data_ptr(), 4096, 3072, 768, st()), reps=20)
+        row = kernel_row("cfg5 matmul_integer 4096x3072x768", us, 19327352832.0, 55836672.0, "hbm")
+        row["mfma_frac"] = round(19327352832.0 / us / 1e6 / PEAK_INT8_MFMA_TOPS, 4)
+        kernels.append(row)
+
+    roofline = None
+    if gemm_us > 0:
+        achieved = gemm_flops / gemm_us / 1e6
+        roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                    "kernel": "gemm_f32_kernel (all GEMM launches of one layer)",
+                    "flop_per_layer": gemm_flops, "us_per_layer": round(gemm_us, 2)}
+
+    # ---- CPU baseline: the oracle's layer on this box's host cores ---------------------------
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        pure_ops.bert_layer(x_host, weights, heads=HEADS)  # warm-up
+        n_cpu, t0 = 0, time.perf_counter()
+        while n_cpu < 8 and time.perf_counter() - t0 < 20.0:
+            pure_ops.bert_layer(x_host, weights, heads=HEADS)
+            n_cpu += 1
+        cpu_ms = (time.perf_counter() - t0) / n_cpu * 1e3
+        cpu_baseline = {"value": round(cpu_ms, 2), "unit": "ms", "cores": cores, "kind": "port",
+                        "sample": f"{n_cpu} runs of the same layer (same seed, B=8 S=128) through the numpy restatement of "
+                                  f"the reference's pure expansions, BLAS matmuls on {cores} threads"}
+
+    result = {
+        "metric": "BERT-base encoder layer latency (B=8, S=128, fp32) via ONNXModel",
+        "value": round(ms_per_step, 5), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE config 3: BERT-base encoder layer, B=8 S=128 H=768 heads=12 FFN=3072, "
+                               "ONNX graph of MatMul/Add/Reshape/Transpose/Div/Softmax/LayerNormalization/Gelu",
+                   "launches_per_step": compiled.num_launches, "replay": "eager" if args.eager else "hip_graph",
+                   "max_rel_err_vs_oracle": err},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

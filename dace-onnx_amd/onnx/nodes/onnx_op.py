@@ -26,6 +26,10 @@ def get_missing_arguments_message(function_name, missing_arguments, argument_typ
         s='' if len(missing_arguments) == 1 else 's', arglist=arglist)
 
 
+def _is_private(connector: str) -> bool:
+    return connector.startswith("_")
+
+
 class ExpansionRefused(NotImplementedError):
     """No implementation available in this build can expand the node.
 
@@ -90,8 +94,12 @@ class ONNXOp(LibraryNode):
                     len(matched), name))
             return matched[0] + number
 
-        sorted_in = sorted(state.in_edges(self), key=lambda e: get_idx(self.schema.inputs, e.dst_conn))
-        sorted_out = sorted(state.out_edges(self), key=lambda e: get_idx(self.schema.outputs, e.src_conn))
+        # connectors with a leading underscore are private to an implementation (operands
+        # folded in by the fusion pass); they are not schema parameters
+        sorted_in = sorted((e for e in state.in_edges(self) if not _is_private(e.dst_conn)),
+                           key=lambda e: get_idx(self.schema.inputs, e.dst_conn))
+        sorted_out = sorted((e for e in state.out_edges(self) if not _is_private(e.src_conn)),
+                            key=lambda e: get_idx(self.schema.outputs, e.src_conn))
         return itertools.chain(zip(sorted_in, itertools.repeat(True)), zip(sorted_out, itertools.repeat(False)))
 
     # ---- validation (onnx_op.py:197-415) ------------------------------------------------
@@ -102,6 +110,8 @@ class ONNXOp(LibraryNode):
         all_connectors = {e.dst_conn for e in in_edges}.union(e.src_conn for e in out_edges)
         if None in all_connectors:
             raise ValueError("Edges to ONNX Ops must not have connector None")
+        in_edges = [e for e in in_edges if not _is_private(e.dst_conn)]
+        out_edges = [e for e in out_edges if not _is_private(e.src_conn)]
 
         known_inputs = {inp.name for inp in self.schema.inputs}
         known_outputs = {outp.name for outp in self.schema.outputs}

@@ -169,10 +169,20 @@ class MI355XMatMul(ONNXForward):
     shared; nothing is copied or transposed."""
 
     @staticmethod
+    def _operands(node, state, sdfg):
+        """Descriptors of A, B, Y as the kernel will address them: the arrays on the
+        edges, or the (shape, strides) views the fusion pass attached."""
+        descs = []
+        for conn, attr, getter in (("A", "_a_view", in_desc_with_name), ("B", "_b_view", in_desc_with_name),
+                                   ("Y", "_y_view", out_desc_with_name)):
+            d = getter(node, state, sdfg, conn)
+            view = getattr(node, attr, None)
+            descs.append(dace.Array(d.dtype, *view) if view else d)
+        return descs
+
+    @staticmethod
     def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
-        A = in_desc_with_name(node, state, sdfg, "A")
-        B = in_desc_with_name(node, state, sdfg, "B")
-        Y = out_desc_with_name(node, state, sdfg, "Y")
+        A, B, Y = MI355XMatMul._operands(node, state, sdfg)
         if len(A.shape) == 1 or len(B.shape) == 1:  # same refusal as PureMatMul (:133-140)
             return False
         if not _is_f32(A, B, Y):
@@ -181,18 +191,7 @@ class MI355XMatMul(ONNXForward):
 
     @staticmethod
     def forward(node, state: SDFGState, sdfg: SDFG):
-        A = in_desc_with_name(node, state, sdfg, "A")
-        B = in_desc_with_name(node, state, sdfg, "B")
-        Y = out_desc_with_name(node, state, sdfg, "Y")
-        a_view = getattr(node, "_a_view", None)  # (shape, strides) set by the fusion pass
-        b_view = getattr(node, "_b_view", None)
-        y_view = getattr(node, "_y_view", None)
-        if a_view:
-            A = dace.Array(A.dtype, *a_view)
-        if b_view:
-            B = dace.Array(B.dtype, *b_view)
-        if y_view:
-            Y = dace.Array(Y.dtype, *y_view)
+        A, B, Y = MI355XMatMul._operands(node, state, sdfg)
         plan = _BatchPlan(A, B, Y)
         if not plan.ok:
             raise ValueError(f"{node.label}: operand layout cannot be expressed as a strided batched GEMM")

@@ -541,10 +541,6 @@ class SDFG:
 # --------------------------------------------------------------------------- executor
 
 
-class _Launch:
-    __slots__ = ("fn", "name", "args", "stream_slots", "ptr_slots", "keepalive")
-
-
 class CompiledSDFG:
     """Executable form of an expanded SDFG: a flat list of kernel launches.
 
@@ -565,14 +561,10 @@ class CompiledSDFG:
         self._lib = _lib.library()  # raises if the HIP library is not built
         self._external = [k for k, d in sdfg.arrays.items() if not d.transient]
         self._written = self._find_written(sdfg)
-        # env maps "array name in the top-level sdfg" -> tensor; nested scopes get their own dict
-        self._launches: typing.List[_Launch] = []
-        self._transients = {}
-        self._aliases = []  # (dst_name, src_name, shape) at top level
-        self._plan = []     # list of (launch, [(arg_index, env_key, offset_bytes)])
+        self._transients = {}   # flattened key -> descriptor
+        self._plan = []         # ("call", node, connector -> key) | ("alias", src key, dst key, dst descriptor)
         self._bound_key = None
         self._graph = None
-        self._static_env = {}
         self._build(sdfg, prefix="", outer_map={})
 
     @staticmethod
@@ -607,9 +599,7 @@ class CompiledSDFG:
                 for e in st.out_edges(n):
                     conn_to_key[e.src_conn] = key_of(e.data.data)
                 if isinstance(n, KernelCall):
-                    self._plan.append(("call", n, conn_to_key, {c: sdfg.arrays[e.data.data] for e in
-                                                             st.in_edges(n) + st.out_edges(n)
-                                                             for c in [e.dst_conn if e.dst is n else e.src_conn]}))
+                    self._plan.append(("call", n, conn_to_key))
                 elif isinstance(n, AliasNode):
                     src_e = [e for e in st.in_edges(n) if e.dst_conn == n.in_conn][0]
                     dst_e = [e for e in st.out_edges(n) if e.src_conn == n.out_conn][0]
@@ -638,7 +628,7 @@ class CompiledSDFG:
                 else:
                     env[dst_key] = src.reshape(dst_desc.shape)  # contiguous -> view
                 continue
-            _, node, conn_to_key, descs = item
+            _, node, conn_to_key = item
             for c, k in conn_to_key.items():
                 if k not in env:
                     d = self._transients[k]
@@ -661,7 +651,7 @@ class CompiledSDFG:
                     args.append(arr)
                 else:
                     args.append(a)
-            launches.append(("call", fn, node.function, args, stream_slots, keep))
+            launches.append(("call", fn, node.function, args, stream_slots, keep, node))
         return env, launches
 
     def _run(self, launches):
@@ -671,7 +661,7 @@ class CompiledSDFG:
             if item[0] == "copy":
                 item[1].copy_(item[2].reshape(item[1].shape))
                 continue
-            _, fn, name, args, stream_slots, _ = item
+            _, fn, name, args, stream_slots, _, _ = item
             for s in stream_slots:
                 args[s] = stream
             status = fn(*args)
@@ -756,3 +746,16 @@ class CompiledSDFG:
     @property
     def num_launches(self):
         return sum(1 for item in self._plan if item[0] == "call")
+
+    def bound_launches(self):
+        """[(KernelCall node, zero-argument callable)] for the currently bound buffers:
+        each callable re-issues that one launch on torch's current stream (profiling)."""
+        import torch
+        if self._bound_key is None:
+            raise RuntimeError("call the compiled SDFG once first")
+        out = []
+        for item in self._launch_list:
+            if item[0] != "call":
+                continue
+            out.append((item[6], (lambda it: (lambda: self._run([it])))(item)))
+        return out

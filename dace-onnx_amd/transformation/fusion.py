@@ -1,5 +1,370 @@
-"""Graph-level fusion before expansion (placeholder: filled in below)."""
+"""Graph-level fusion of ONNX library nodes before expansion.
+
+The reference fuses at graph level too, with pattern transformations over the
+SDFG: ``PadConvFusion`` folds a Pad into the Conv that follows
+(``daceml/transformation/pad_conv_fusion.py:13-95``), ``TaskletFusion`` merges
+elementwise tasklets (``tasklet_fusion.py:35``), ``ReshapeElimination`` drops
+Reshapes. Here the patterns are the ones that remove HBM round trips around a
+contraction, because the MFMA kernels can absorb them:
+
+===========================================  =====================================
+pattern (every intermediate single-use)      becomes
+===========================================  =====================================
+MatMul -> Div/Mul by a constant scalar       MatMul with ``_alpha``
+MatMul -> Add(1-D bias over N)               MatMul with input connector ``_bias``
+MatMul/Gemm -> Relu | Gelu                   ``_activation``
+MatMul -> Add(tensor of the output's shape)  input connector ``_residual``
+Conv -> Relu                                 ``_activation = "relu"``
+X -> Reshape/Transpose chain -> MatMul       MatMul reads X through ``_a_view`` /
+                                             ``_b_view`` (shape, strides)
+MatMul -> Transpose -> Reshape               MatMul writes the final array through
+                                             ``_y_view``
+===========================================  =====================================
+
+The annotations are private attributes / connectors (leading underscore) that
+the ``"mi355x"`` MatMul, Gemm and Conv expansions understand; the reference
+passes per-node tuning the same way (``node._algorithm``,
+``cudnn_implementations.py:251-254``). Order inside the kernel epilogue is fixed:
+alpha, bias, activation, residual -- a pattern is only folded when it respects it.
+Nodes left without consumers are removed afterwards.
+"""
+import logging
+import typing
+
+import numpy as np
+
+from ..sdfg import SDFG, SDFGState, AccessNode, Array, _contiguous_strides
+
+log = logging.getLogger(__name__)
 
 
-def fuse_onnx_graph(sdfg) -> int:
-    return 0
+# ----------------------------------------------------------------------------- graph helpers
+def _is_op(node, *names):
+    schema = getattr(node, "schema", None)
+    return schema is not None and schema.name in names
+
+
+def _in_edge(state, node, conn):
+    c = [e for e in state.in_edges(node) if e.dst_conn == conn]
+    return c[0] if len(c) == 1 else None
+
+
+def _out_edge(state, node, conn):
+    c = [e for e in state.out_edges(node) if e.src_conn == conn]
+    return c[0] if len(c) == 1 else None
+
+
+def _single_consumer(sdfg, state, access: AccessNode):
+    """The only reader of a transient that is written once; None otherwise."""
+    desc = sdfg.arrays[access.data]
+    if not desc.transient or len(state.in_edges(access)) != 1:
+        return None
+    outs = state.out_edges(access)
+    if len(outs) != 1:
+        return None
+    # no other access node of the same array may read it
+    for n in state.nodes():
+        if isinstance(n, AccessNode) and n is not access and n.data == access.data:
+            return None
+    return outs[0]
+
+
+def _producer(state, access: AccessNode):
+    ins = state.in_edges(access)
+    return ins[0] if len(ins) == 1 else None
+
+
+def _constant_value(sdfg, name) -> typing.Optional[np.ndarray]:
+    model = getattr(sdfg, "_parent_onnx_model", None)
+    if model is None:
+        return None
+    w = model.clean_weights.get(name)
+    return None if w is None else w.detach().cpu().numpy()
+
+
+def _reshape_strides(shape, strides, new_shape):
+    """Strides that view (shape, strides) as ``new_shape`` without copying, or None
+    (the no-copy reshape rule of numpy)."""
+    old = [(s, st) for s, st in zip(shape, strides) if s != 1]
+    new_strides = [0] * len(new_shape)
+    oi = 0
+    ni = 0
+    while ni < len(new_shape):
+        if new_shape[ni] == 1:
+            new_strides[ni] = 0
+            ni += 1
+            continue
+        if oi >= len(old):
+            return None
+        # grow a group of old dims and a group of new dims until their sizes match
+        o_size, n_size = old[oi][0], new_shape[ni]
+        o_end, n_end = oi + 1, ni + 1
+        while o_size != n_size:
+            if o_size < n_size:
+                if o_end >= len(old):
+                    return None
+                o_size *= old[o_end][0]
+                o_end += 1
+            else:
+                while n_end < len(new_shape) and new_shape[n_end] == 1:
+                    n_end += 1
+                if n_end >= len(new_shape):
+                    return None
+                n_size *= new_shape[n_end]
+                n_end += 1
+        # the old group must be contiguous within itself
+        for k in range(oi, o_end - 1):
+            if old[k][1] != old[k + 1][1] * old[k + 1][0]:
+                return None
+        st = old[o_end - 1][1]
+        for k in range(n_end - 1, ni - 1, -1):
+            new_strides[k] = st if new_shape[k] != 1 else 0
+            st *= new_shape[k]
+        oi, ni = o_end, n_end
+    if oi != len(old):
+        return None
+    return new_strides
+
+
+# ----------------------------------------------------------------------------- elementwise folds
+def _replace_output(sdfg, state, node, out_conn, folded_node, folded_out_conn):
+    """``node`` takes over the output of ``folded_node``; the intermediate array and
+    ``folded_node`` disappear."""
+    mid_edge = _out_edge(state, node, out_conn)
+    mid_access = mid_edge.dst
+    final_edge = _out_edge(state, folded_node, folded_out_conn)
+    state.remove_edge(mid_edge)
+    state.add_edge(node, out_conn, final_edge.dst, None, final_edge.data)
+    state.remove_node(folded_node)
+    state.remove_node(mid_access)
+    del sdfg.arrays[mid_access.data]
+
+
+def _fold_into_contractions(sdfg: SDFG, state: SDFGState) -> int:
+    folded = 0
+    changed = True
+    while changed:
+        changed = False
+        for node in state.nodes():
+            if not _is_op(node, "MatMul", "Gemm", "Conv"):
+                continue
+            out_e = _out_edge(state, node, "Y")
+            if out_e is None or not isinstance(out_e.dst, AccessNode):
+                continue
+            use = _single_consumer(sdfg, state, out_e.dst)
+            if use is None:
+                continue
+            nxt = use.dst
+            ydesc = sdfg.arrays[out_e.dst.data]
+            has_bias = _in_edge(state, node, "_bias") is not None
+            has_res = _in_edge(state, node, "_residual") is not None
+            act = getattr(node, "_activation", None)
+
+            # ---- scalar scale -> alpha (must come first in the epilogue)
+            if _is_op(node, "MatMul") and _is_op(nxt, "Div", "Mul") and use.dst_conn == "A" \
+                    and not (has_bias or has_res or act):
+                other = _in_edge(state, nxt, "B")
+                val = _constant_value(sdfg, other.src.data) if other is not None else None
+                if val is not None and val.size == 1 and tuple(sdfg.arrays[_out_edge(state, nxt, "C").dst.data].shape) == tuple(ydesc.shape):
+                    v = float(val.reshape(-1)[0])
+                    node._alpha = getattr(node, "_alpha", 1.0) * ((1.0 / v) if _is_op(nxt, "Div") else v)
+                    _replace_output(sdfg, state, node, "Y", nxt, "C")
+                    folded += 1
+                    changed = True
+                    break
+            # ---- bias over the last dimension
+            if _is_op(node, "MatMul") and _is_op(nxt, "Add") and not (has_bias or has_res or act):
+                other_conn = "B" if use.dst_conn == "A" else "A"
+                other = _in_edge(state, nxt, other_conn)
+                if other is not None:
+                    od = sdfg.arrays[other.src.data]
+                    n_dim = ydesc.shape[-1]
+                    out_shape = tuple(sdfg.arrays[_out_edge(state, nxt, "C").dst.data].shape)
+                    if od.total_size == n_dim and od.shape and od.shape[-1] == n_dim and od.is_contiguous() \
+                            and out_shape == tuple(ydesc.shape) and n_dim > 1:
+                        node.add_in_connector("_bias")
+                        state.add_edge(other.src, None, node, "_bias", other.data)
+                        _replace_output(sdfg, state, node, "Y", nxt, "C")
+                        folded += 1
+                        changed = True
+                        break
+            # ---- activation
+            if _is_op(nxt, "Relu", "Gelu") and not has_res and act is None:
+                is_gelu = _is_op(nxt, "Gelu")
+                if (not is_gelu or ((nxt.approximate or "none") == "none" and not _is_op(node, "Conv"))):
+                    node._activation = "gelu" if is_gelu else "relu"
+                    _replace_output(sdfg, state, node, "Y", nxt, "Y")
+                    folded += 1
+                    changed = True
+                    break
+            # ---- residual (last in the epilogue)
+            if _is_op(node, "MatMul") and _is_op(nxt, "Add") and not has_res:
+                other_conn = "B" if use.dst_conn == "A" else "A"
+                other = _in_edge(state, nxt, other_conn)
+                if other is not None:
+                    od = sdfg.arrays[other.src.data]
+                    out_shape = tuple(sdfg.arrays[_out_edge(state, nxt, "C").dst.data].shape)
+                    if tuple(od.shape) == tuple(ydesc.shape) == out_shape and od.is_contiguous() and ydesc.is_contiguous():
+                        node.add_in_connector("_residual")
+                        state.add_edge(other.src, None, node, "_residual", other.data)
+                        _replace_output(sdfg, state, node, "Y", nxt, "C")
+                        folded += 1
+                        changed = True
+                        break
+    return folded
+
+
+# ----------------------------------------------------------------------------- view folds
+def _input_view(sdfg, state, access: AccessNode):
+    """Walk back through Reshape/Transpose producers of ``access``. Returns
+    (source access node, shape, strides) describing ``access`` as a strided view
+    of the source array, or None when there is nothing to fold."""
+    chain = []
+    cur = access
+    while True:
+        prod = _producer(state, cur)
+        if prod is None or not sdfg.arrays[cur.data].transient:
+            break
+        n = prod.src
+        if _is_op(n, "Transpose"):
+            chain.append(("T", n))
+            cur = _in_edge(state, n, "data").src
+        elif _is_op(n, "Reshape"):
+            chain.append(("R", n))
+            cur = _in_edge(state, n, "data").src
+        else:
+            break
+        if not isinstance(cur, AccessNode):
+            return None
+    if not chain:
+        return None
+    src = sdfg.arrays[cur.data]
+    if not src.is_contiguous():
+        return None
+    shape, strides = list(src.shape), list(src.strides)
+    for kind, n in reversed(chain):
+        if kind == "T":
+            perm = list(n.perm) if n.perm is not None else list(reversed(range(len(shape))))
+            shape, strides = [shape[p] for p in perm], [strides[p] for p in perm]
+        else:
+            new_shape = list(sdfg.arrays[_out_edge(state, n, "reshaped").dst.data].shape)
+            new_strides = _reshape_strides(shape, strides, new_shape)
+            if new_strides is None:
+                return None
+            shape, strides = new_shape, new_strides
+    if tuple(shape) != tuple(sdfg.arrays[access.data].shape):
+        return None
+    return cur, shape, strides
+
+
+def _fold_views(sdfg: SDFG, state: SDFGState) -> int:
+    from ..onnx.op_implementations.mi355x_implementations import _BatchPlan
+    folded = 0
+    for node in state.nodes():
+        if not _is_op(node, "MatMul"):
+            continue
+        a_e, b_e, y_e = _in_edge(state, node, "A"), _in_edge(state, node, "B"), _out_edge(state, node, "Y")
+        if a_e is None or b_e is None or y_e is None:
+            continue
+
+        def desc_of(edge, view):
+            d = sdfg.arrays[edge.data.data]
+            return Array(d.dtype, *view) if view else d
+
+        views = {"A": getattr(node, "_a_view", None), "B": getattr(node, "_b_view", None),
+                 "Y": getattr(node, "_y_view", None)}
+        # ---- inputs: read through Reshape/Transpose chains
+        for conn, edge, attr in (("A", a_e, "_a_view"), ("B", b_e, "_b_view")):
+            if views[conn] is not None or not isinstance(edge.src, AccessNode):
+                continue
+            found = _input_view(sdfg, state, edge.src)
+            if found is None:
+                continue
+            src_access, shape, strides = found
+            trial = dict(views)
+            trial[conn] = (shape, strides)
+            plan = _BatchPlan(Array(sdfg.arrays[src_access.data].dtype, *trial["A"]) if trial["A"] else sdfg.arrays[a_e.data.data],
+                              Array(sdfg.arrays[src_access.data].dtype, *trial["B"]) if trial["B"] else sdfg.arrays[b_e.data.data],
+                              desc_of(y_e, trial["Y"]))
+            if not plan.ok:
+                continue
+            state.remove_edge(edge)
+            new_edge = state.add_edge(src_access, None, node, conn, sdfg.make_array_memlet(src_access.data))
+            setattr(node, attr, (shape, strides))
+            views[conn] = (shape, strides)
+            if conn == "A":
+                a_e = new_edge
+            else:
+                b_e = new_edge
+            folded += 1
+        # ---- output: write through Transpose (-> Reshape)
+        if views["Y"] is None and _in_edge(state, node, "_bias") is None and _in_edge(state, node, "_residual") is None \
+                and getattr(node, "_activation", None) is None and isinstance(y_e.dst, AccessNode):
+            use = _single_consumer(sdfg, state, y_e.dst)
+            if use is not None and _is_op(use.dst, "Transpose"):
+                tnode = use.dst
+                ydesc = sdfg.arrays[y_e.dst.data]
+                perm = list(tnode.perm) if tnode.perm is not None else list(reversed(range(len(ydesc.shape))))
+                t_access = _out_edge(state, tnode, "transposed").dst
+                t_strides = _contiguous_strides(sdfg.arrays[t_access.data].shape)
+                y_strides = [0] * len(perm)
+                for k, p in enumerate(perm):
+                    y_strides[p] = t_strides[k]
+                final_access, drop = t_access, [tnode]
+                use2 = _single_consumer(sdfg, state, t_access)
+                if use2 is not None and _is_op(use2.dst, "Reshape") and use2.dst_conn == "data":
+                    final_access = _out_edge(state, use2.dst, "reshaped").dst
+                    drop.append(use2.dst)
+                if ydesc.is_contiguous() and sdfg.arrays[final_access.data].is_contiguous() and y_strides[-1] == 1:
+                    view = (list(ydesc.shape), y_strides)
+                    plan = _BatchPlan(desc_of(a_e, views["A"]), desc_of(b_e, views["B"]), Array(ydesc.dtype, *view))
+                    if plan.ok:
+                        mids = [y_e.dst] + ([t_access] if final_access is not t_access else [])
+                        state.remove_edge(y_e)
+                        state.add_edge(node, "Y", final_access, None, sdfg.make_array_memlet(final_access.data))
+                        for d in drop:
+                            state.remove_node(d)
+                        for m in mids:
+                            state.remove_node(m)
+                            del sdfg.arrays[m.data]
+                        node._y_view = view
+                        folded += 1
+    return folded
+
+
+def _remove_dead_nodes(sdfg: SDFG, state: SDFGState) -> int:
+    """Drop nodes whose outputs nobody reads (left behind by the view folds)."""
+    removed = 0
+    changed = True
+    while changed:
+        changed = False
+        for n in state.nodes():
+            if isinstance(n, AccessNode):
+                desc = sdfg.arrays.get(n.data)
+                if desc is not None and desc.transient and not state.out_edges(n) and state.in_edges(n):
+                    prod = state.in_edges(n)[0].src
+                    # only pure data-movement nodes are dropped; anything else would be a graph bug
+                    if _is_op(prod, "Transpose", "Reshape", "Identity", "Flatten") and len(state.out_edges(prod)) == 1:
+                        state.remove_node(prod)
+                        state.remove_node(n)
+                        del sdfg.arrays[n.data]
+                        removed += 1
+                        changed = True
+                        break
+                elif not state.in_edges(n) and not state.out_edges(n):
+                    state.remove_node(n)
+                    changed = True
+                    break
+    return removed
+
+
+def fuse_onnx_graph(sdfg: SDFG) -> int:
+    """Apply every fusion pattern to every state; returns the number of folds."""
+    total = 0
+    for state in sdfg.nodes():
+        total += _fold_into_contractions(sdfg, state)
+        total += _fold_views(sdfg, state)
+        _remove_dead_nodes(sdfg, state)
+    if total:
+        log.info("fused %d patterns in SDFG %s", total, sdfg.name)
+    return total
