@@ -24,23 +24,11 @@
 //     range of tiles instead of every eighth tile.
 #include "common.h"
 #include "gemm_tile.h"
+#include "gemm_args.h"
 
 #include <stdlib.h>
 
 namespace mi355x {
-
-struct GemmArgs {
-    const float* A; const float* B; float* C; const float* bias; const float* residual;
-    int64_t batch1;
-    int64_t M, N, K;
-    int64_t a_sb0, a_sb1, a_sm, a_sk;
-    int64_t b_sb0, b_sb1, b_sk, b_sn;
-    int64_t c_sb0, c_sb1, c_sm;
-    int64_t r_sb0, r_sb1, r_sm;
-    int64_t tiles_m, tiles_n, nwg;
-    float alpha;
-    int epi;
-};
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f32_kernel(GemmArgs p) {
@@ -225,7 +213,7 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
 
     GemmArgs p;
     p.A = A; p.B = B; p.C = C; p.bias = bias; p.residual = residual;
-    p.batch1 = batch1; p.M = M; p.N = N; p.K = K;
+    p.batch = batch; p.batch1 = batch1; p.M = M; p.N = N; p.K = K;
     p.a_sb0 = a_strides[0]; p.a_sb1 = a_strides[1]; p.a_sm = a_strides[2]; p.a_sk = a_strides[3];
     p.b_sb0 = b_strides[0]; p.b_sb1 = b_strides[1]; p.b_sk = b_strides[2]; p.b_sn = b_strides[3];
     p.c_sb0 = c_strides[0]; p.c_sb1 = c_strides[1]; p.c_sm = c_strides[2];
@@ -248,6 +236,10 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
 
     int cus = mi355x_device_cu_count();
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "gemm: no usable HIP device");
+    // both operands contiguous along k (activations x pre-transposed weights, Q K^T):
+    // the dedicated kernel reads every MFMA fragment with 16-byte accesses
+    if (a_kc && b_kc && vec && !getenv("MI355X_GEMM_CONFIG") && launch_gemm_f32_nt(p, cus, static_cast<hipStream_t>(stream)))
+        return check_launch("gemm_f32_nt_kernel");
     const int cfg = choose_config(batch, M, N, K, cus);
     const TileConfig& tc = kConfigs[cfg];
     p.tiles_m = ceil_div(M, tc.bm);
