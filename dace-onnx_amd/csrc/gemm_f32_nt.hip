@@ -50,7 +50,8 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     constexpr int BM = NT_BM, BN = 16 * TN, BK = NT_BK, RING = NT_RING;
     constexpr int B_VECS = BN * (BK / 4);                       // 16-byte vectors of one B tile
     constexpr int B_PER_T = (B_VECS + NT_THREADS - 1) / NT_THREADS;
-    constexpr int STAGE = BN * NT_PITCH;                        // floats per LDS buffer
+    constexpr int B_ROWS = B_PER_T * NT_THREADS / (BK / 4);     // rows incl. the ones only written as padding
+    constexpr int STAGE = B_ROWS * NT_PITCH;                    // floats per LDS buffer
     constexpr int RED = BM * BN;                                // partial sums of k-split group 1
     constexpr int LDS_FLOATS = NT_STAGES * STAGE > RED ? NT_STAGES * STAGE : RED;
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
@@ -99,10 +100,10 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
             dst[it] = *reinterpret_cast<const f32x4*>(b_ptr[it] + (int64_t)kt * BK);
     };
     auto store_b = [&](const f32x4 (&src)[B_PER_T], int stage) {
+        // every thread stores (rows >= BN are padding): no branch in the step body
 #pragma unroll
         for (int it = 0; it < B_PER_T; ++it)
-            if (B_VECS % NT_THREADS == 0 || tid + it * NT_THREADS < B_VECS)
-                *reinterpret_cast<f32x4*>(lds + stage * STAGE + b_lds[it]) = src[it];
+            *reinterpret_cast<f32x4*>(lds + stage * STAGE + b_lds[it]) = src[it];
     };
     auto read_b = [&](f32x4 (&dst)[TN], int stage) {
 #pragma unroll
@@ -110,20 +111,39 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
             dst[j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * NT_PITCH + 16 * ks + 4 * lq);
     };
 
-    auto tile_step = [&](auto r_tag, auto pre_tag, auto wr_tag, auto nxt_tag, int kt) {
+    auto tile_step = [&](auto r_tag, auto pre_tag, auto prea_tag, auto wr_tag, auto nxt_tag, int kt) {
         constexpr int r = decltype(r_tag)::value;
-        constexpr bool PRE = decltype(pre_tag)::value, WR = decltype(wr_tag)::value, NXT = decltype(nxt_tag)::value;
+        constexpr bool PRE = decltype(pre_tag)::value, PRE_A = decltype(prea_tag)::value;
+        constexpr bool WR = decltype(wr_tag)::value, NXT = decltype(nxt_tag)::value;
+        // The step's six memory instructions are spread between its MFMAs: issued
+        // as one burst after the barrier they queue behind the other waves' requests
+        // in the texture-address and LDS units and stall MFMA issue (measured: a
+        // 16-byte LDS write costs a wave ~60 cycles of issue time, a global load up to
+        // ~140 when eight waves issue together).
         if constexpr (PRE) load_b(rb[r], kt + RING);                         // slot r left for LDS two steps ago
+        if constexpr (PRE_A) load_a(ra[(r + RING - 1) % RING], kt + RING - 1);  // fragment consumed in the previous step
         if constexpr (WR) store_b(rb[(r + 2) % RING], (r + 2) % NT_STAGES);  // tile kt + 2
         if constexpr (NXT) read_b(bf[(r + 1) & 1], (r + 1) % NT_STAGES);     // tile kt + 1, already visible
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[r & 1][j][s], ra[r][s], acc[j], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (PRE) load_a(ra[r], kt + RING);                         // its fragment has just been consumed
+        // order: LDS traffic first, one instruction after each of the first MFMAs (it must
+        // be complete at the barrier), the global loads later in the step
+        constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
+        __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(DS_RD, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(MFMA, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(VMEM_RD, B_PER_T, 0);
+        __builtin_amdgcn_sched_group_barrier(MFMA, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(VMEM_RD, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(MFMA, 4 * TN, 0);
         __syncthreads();
     };
 
@@ -142,7 +162,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     int kt0 = 0;
     for (; kt0 + 2 * RING <= ktiles; kt0 += RING) {  // steady state: branch-free body
         nt_static_for<RING>([&](auto r_tag) {
-            tile_step(r_tag, std::true_type{}, std::true_type{}, std::true_type{}, kt0 + decltype(r_tag)::value);
+            tile_step(r_tag, std::true_type{}, std::true_type{}, std::true_type{}, std::true_type{}, kt0 + decltype(r_tag)::value);
         });
     }
     for (; kt0 < ktiles; kt0 += RING) {              // tail: look-aheads switch off one by one
@@ -151,10 +171,11 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
             if (kt < ktiles) {
                 constexpr std::true_type T{};
                 constexpr std::false_type F{};
-                if (kt + RING < ktiles) tile_step(r_tag, T, T, T, kt);
-                else if (kt + 2 < ktiles) tile_step(r_tag, F, T, T, kt);
-                else if (kt + 1 < ktiles) tile_step(r_tag, F, F, T, kt);
-                else tile_step(r_tag, F, F, F, kt);
+                if (kt + RING < ktiles) tile_step(r_tag, T, T, T, T, kt);
+                else if (kt + RING == ktiles) tile_step(r_tag, F, T, T, T, kt);
+                else if (kt + 2 < ktiles) tile_step(r_tag, F, F, T, T, kt);
+                else if (kt + 1 < ktiles) tile_step(r_tag, F, F, F, T, kt);
+                else tile_step(r_tag, F, F, F, F, kt);
             }
         });
     }
