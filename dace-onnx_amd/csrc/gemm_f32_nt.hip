@@ -27,6 +27,7 @@
 #include "gemm_tile.h"
 #include "gemm_args.h"
 
+#include <stdlib.h>
 #include <type_traits>
 #include <utility>
 
@@ -42,24 +43,29 @@ __device__ __forceinline__ void nt_static_for(F&& f) {
     nt_static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
 
-constexpr int NT_BM = 64, NT_BK = 32, NT_THREADS = 512, NT_RING = 6, NT_STAGES = 3;
+constexpr int NT_BK = 32, NT_THREADS = 512, NT_RING = 6, NT_STAGES = 3;
 constexpr int NT_PITCH = NT_BK + LDS_PAD;
 
-template <int TN>
+// TN: 16-column MFMA tiles per wave (BN = 16 TN). WAVES_M wave rows of 16 rows each
+// (BM = 16 WAVES_M) times KSPLIT k-split groups make the 8 waves of a workgroup:
+// (4, 2) for problems with few tiles, (8, 1) for 128-row tiles without a reduction.
+template <int TN, int WAVES_M, int KSPLIT>
 __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
-    constexpr int BM = NT_BM, BN = 16 * TN, BK = NT_BK, RING = NT_RING;
+    static_assert(WAVES_M * KSPLIT * WAVE == NT_THREADS, "8 waves per workgroup");
+    constexpr int BM = 16 * WAVES_M, BN = 16 * TN, BK = NT_BK, RING = NT_RING;
+    constexpr int NC = (BK / 16) / KSPLIT;  // 16-k chunks of a tile this wave multiplies
     constexpr int B_VECS = BN * (BK / 4);                       // 16-byte vectors of one B tile
     constexpr int B_PER_T = (B_VECS + NT_THREADS - 1) / NT_THREADS;
     constexpr int B_ROWS = B_PER_T * NT_THREADS / (BK / 4);     // rows incl. the ones only written as padding
     constexpr int STAGE = B_ROWS * NT_PITCH;                    // floats per LDS buffer
-    constexpr int RED = BM * BN;                                // partial sums of k-split group 1
+    constexpr int RED = (KSPLIT - 1) * BM * BN;                 // partial sums of k-split group 1
     constexpr int LDS_FLOATS = NT_STAGES * STAGE > RED ? NT_STAGES * STAGE : RED;
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
 
     const int tid = threadIdx.x;
     const int lane = tid % WAVE, wave = tid / WAVE;
     const int li = lane % 16, lq = lane / 16;
-    const int wm = wave % 4, ks = wave / 4;   // wave row, k-split group
+    const int wm = wave % WAVES_M, ks = wave / WAVES_M;   // wave row, k-split group
 
     const int64_t logical = xcd_remap(blockIdx.x, p.nwg);
     const int64_t tiles_per_batch = p.tiles_m * p.tiles_n;
@@ -68,7 +74,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     const int64_t m0 = (t / p.tiles_n) * BM, n0 = (t % p.tiles_n) * BN;
 
     // this lane's A fragment source: row m (clamped into the matrix), 4 floats at
-    // k = 32*kt + 16*ks + 4*lq
+    // k = 32*kt + 16*(c*KSPLIT + ks) + 4*lq for its chunks c
     int64_t am = m0 + 16 * wm + li;
     am = am < p.M ? am : p.M - 1;
     const float* __restrict__ a_ptr = p.A + b0 * p.a_sb0 + b1 * p.a_sb1 + am * p.a_sm + 16 * ks + 4 * lq;
@@ -89,15 +95,21 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    f32x4 ra[RING];            // A fragment of tile t in slot t % RING
+    const int ktiles = (int)(p.K / BK);  // K % 32 == 0 is a launch precondition
+    const int last_tile = ktiles - 1;
+    f32x4 ra[RING][NC];        // A fragments of tile t in slot t % RING
     f32x4 rb[RING][B_PER_T];   // B tile slice of tile t in slot t % RING
-    f32x4 bf[2][TN];           // B fragments of tile t in set t % 2
+    f32x4 bf[2][TN];           // B fragments of the wave's g-th chunk in set g % 2 (g counts across tiles)
 
-    auto load_a = [&](f32x4& dst, int kt) { dst = *reinterpret_cast<const f32x4*>(a_ptr + (int64_t)kt * BK); };
+    auto load_a = [&](f32x4 (&dst)[NC], int kt) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+            dst[c] = *reinterpret_cast<const f32x4*>(a_ptr + (int64_t)(kt < last_tile ? kt : last_tile) * BK + 16 * c * KSPLIT);
+    };
     auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt) {
 #pragma unroll
         for (int it = 0; it < B_PER_T; ++it)
-            dst[it] = *reinterpret_cast<const f32x4*>(b_ptr[it] + (int64_t)kt * BK);
+            dst[it] = *reinterpret_cast<const f32x4*>(b_ptr[it] + (int64_t)(kt < last_tile ? kt : last_tile) * BK);
     };
     auto store_b = [&](const f32x4 (&src)[B_PER_T], int stage) {
         // every thread stores (rows >= BN are padding): no branch in the step body
@@ -105,10 +117,11 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         for (int it = 0; it < B_PER_T; ++it)
             *reinterpret_cast<f32x4*>(lds + stage * STAGE + b_lds[it]) = src[it];
     };
-    auto read_b = [&](f32x4 (&dst)[TN], int stage) {
+    auto read_b = [&](f32x4 (&dst)[TN], int stage, int c) {
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-            dst[j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * NT_PITCH + 16 * ks + 4 * lq);
+            dst[j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * NT_PITCH +
+                                                     16 * (c * KSPLIT + ks) + 4 * lq);
     };
 
     auto tile_step = [&](auto r_tag, auto pre_tag, auto prea_tag, auto wr_tag, auto nxt_tag, int kt) {
@@ -121,17 +134,27 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         // 16-byte LDS write costs a wave ~60 cycles of issue time, a global load up to
         // ~140 when eight waves issue together).
         if constexpr (PRE) load_b(rb[r], kt + RING);                         // slot r left for LDS two steps ago
-        if constexpr (PRE_A) load_a(ra[(r + RING - 1) % RING], kt + RING - 1);  // fragment consumed in the previous step
+        if constexpr (PRE_A) load_a(ra[(r + RING - 1) % RING], kt + RING - 1);  // fragments consumed in the previous step
         if constexpr (WR) store_b(rb[(r + 2) % RING], (r + 2) % NT_STAGES);  // tile kt + 2
-        if constexpr (NXT) read_b(bf[(r + 1) & 1], (r + 1) % NT_STAGES);     // tile kt + 1, already visible
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[r & 1][j][s], ra[r][s], acc[j], 0, 0, 0);
-        // order: LDS traffic first, one instruction after each of the first MFMAs (it must
-        // be complete at the barrier), the global loads later in the step
         constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            constexpr int g0 = (r * NC) & 1;
+            const int cur = (g0 + c) & 1;
+            // fragments of the next chunk: same tile, or chunk 0 of tile kt + 1 (visible since the last barrier)
+            if (c + 1 < NC) read_b(bf[cur ^ 1], r % NT_STAGES, c + 1);
+            else if constexpr (NXT) read_b(bf[cur ^ 1], (r + 1) % NT_STAGES, 0);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[cur][j][s], ra[r][c][s], acc[j], 0, 0, 0);
+        }
+        // Issue order inside the step. A wave's memory instructions are spread between
+        // its MFMAs: issued as one burst after the barrier they queue behind the other
+        // waves' requests in the LDS and texture-address units and hold up MFMA issue.
+        // LDS traffic comes first (it must have completed at the barrier), the global
+        // loads later.
         __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
         __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
 #pragma unroll
@@ -142,54 +165,53 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         __builtin_amdgcn_sched_group_barrier(MFMA, 2, 0);
         __builtin_amdgcn_sched_group_barrier(VMEM_RD, B_PER_T, 0);
         __builtin_amdgcn_sched_group_barrier(MFMA, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(VMEM_RD, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(MFMA, 4 * TN, 0);
+        __builtin_amdgcn_sched_group_barrier(VMEM_RD, NC, 0);
+        if constexpr (NC == 2) {
+            __builtin_amdgcn_sched_group_barrier(MFMA, 3 * TN - 5, 0);  // rest of chunk 0
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DS_RD, 1, 0);
+            }
+        }
+        __builtin_amdgcn_sched_group_barrier(MFMA, 4 * TN * NC, 0);
         __syncthreads();
     };
 
-    const int ktiles = (int)(p.K / BK);  // K % 32 == 0 is a launch precondition
 #pragma unroll
-    for (int r = 0; r < RING; ++r)
-        if (r < ktiles) {
-            load_a(ra[r], r);
-            load_b(rb[r], r);
-        }
-    store_b(rb[0], 0);
-    if (ktiles > 1) store_b(rb[1], 1);
-    __syncthreads();
-    if (ktiles > 0) read_b(bf[0], 0);
-
-    int kt0 = 0;
-    for (; kt0 + 2 * RING <= ktiles; kt0 += RING) {  // steady state: branch-free body
-        nt_static_for<RING>([&](auto r_tag) {
-            tile_step(r_tag, std::true_type{}, std::true_type{}, std::true_type{}, std::true_type{}, kt0 + decltype(r_tag)::value);
-        });
+    for (int r = 0; r < RING; ++r) {  // tiles beyond the last are clamped: no branch
+        load_a(ra[r], r);
+        load_b(rb[r], r);
     }
-    for (; kt0 < ktiles; kt0 += RING) {              // tail: look-aheads switch off one by one
+    store_b(rb[0], 0);
+    store_b(rb[1], 1);
+    __syncthreads();
+    read_b(bf[0], 0, 0);
+
+    // One code path for every tile: near the end of K the look-aheads are not switched
+    // off but clamped to the last tile (they re-read data that is already in cache and
+    // write LDS buffers nobody reads any more), so the step body stays branch-free
+    // and the compiler's s_waitcnt counts stay exact from the first tile to the last.
+    for (int kt0 = 0; kt0 < ktiles; kt0 += RING) {
         nt_static_for<RING>([&](auto r_tag) {
             const int kt = kt0 + decltype(r_tag)::value;
-            if (kt < ktiles) {
-                constexpr std::true_type T{};
-                constexpr std::false_type F{};
-                if (kt + RING < ktiles) tile_step(r_tag, T, T, T, T, kt);
-                else if (kt + RING == ktiles) tile_step(r_tag, F, T, T, T, kt);
-                else if (kt + 2 < ktiles) tile_step(r_tag, F, F, T, T, kt);
-                else if (kt + 1 < ktiles) tile_step(r_tag, F, F, F, T, kt);
-                else tile_step(r_tag, F, F, F, F, kt);
-            }
+            if (kt < ktiles)  // uniform; only the last group can be partial
+                tile_step(r_tag, std::true_type{}, std::true_type{}, std::true_type{}, std::true_type{}, kt);
         });
     }
 
     // k-split group 1 hands its partial sums to group 0 through LDS
-    f32x4* red = reinterpret_cast<f32x4*>(lds);
-    if (ks == 1) {
+    if constexpr (KSPLIT == 2) {
+        f32x4* red = reinterpret_cast<f32x4*>(lds);
+        if (ks == 1) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) red[(wm * TN + j) * WAVE + lane] = acc[j];
+            for (int j = 0; j < TN; ++j) red[(wm * TN + j) * WAVE + lane] = acc[j];
+        }
+        __syncthreads();
+        if (ks == 1) return;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[j] += red[(wm * TN + j) * WAVE + lane];
     }
-    __syncthreads();
-    if (ks == 1) return;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[j] += red[(wm * TN + j) * WAVE + lane];
 
     // epilogue: acc[j][r] = C[m0 + 16*wm + li][n0 + 16*j + 4*lq + r]
     const int64_t m = m0 + 16 * wm + li;
@@ -216,23 +238,27 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
 // and N a multiple of 4. Additionally needed here: K a multiple of the 32-k tile.
 bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.K % NT_BK != 0 || p.K == 0) return false;
-    // TN = 3 (48 columns) when it tiles N exactly or gives a fuller last wave of
-    // workgroups than 64-column tiles do
-    const int64_t tm = ceil_div(p.M, NT_BM);
-    auto waste = [&](int bn) {
-        const int64_t nwg = p.batch * tm * ceil_div(p.N, bn);
-        const int64_t rounds = ceil_div(nwg, (int64_t)cus);
-        return (double)(rounds * cus) * bn;  // column-slots of work the machine is occupied for
-    };
-    const bool use48 = waste(48) <= waste(64);
-    const int bn = use48 ? 48 : 64;
-    p.tiles_m = tm;
-    p.tiles_n = ceil_div(p.N, bn);
+    // Candidates: 64x48 and 64x64 tiles with two k-split groups, 128x96 tiles without.
+    // Cost ~ rounds of workgroups over the CUs x tile area, the large tile discounted
+    // for needing half the L2 traffic per FLOP and no reduction.
+    struct Cand { int bm, bn; double weight; };
+    const Cand cands[] = {{64, 48, 1.0}, {64, 64, 1.0}, {128, 96, 0.8}};
+    int best = 0;
+    double best_cost = 1e300;
+    const char* force = getenv("MI355X_GEMM_NT_BN");
+    for (int c = 0; c < 3; ++c) {
+        const int64_t nwg = p.batch * ceil_div(p.M, cands[c].bm) * ceil_div(p.N, cands[c].bn);
+        const double cost = (double)ceil_div(nwg, (int64_t)cus) * cands[c].bm * cands[c].bn * cands[c].weight;
+        if (force ? atoi(force) == cands[c].bn : cost < best_cost) { best = c; best_cost = cost; if (force) break; }
+    }
+    p.tiles_m = ceil_div(p.M, cands[best].bm);
+    p.tiles_n = ceil_div(p.N, cands[best].bn);
     p.nwg = p.batch * p.tiles_m * p.tiles_n;
     if (p.nwg >= ((int64_t)1 << 31)) return false;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
-    if (use48) hipLaunchKernelGGL(gemm_f32_nt_kernel<3>, grid, block, 0, stream, p);
-    else hipLaunchKernelGGL(gemm_f32_nt_kernel<4>, grid, block, 0, stream, p);
+    if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
+    else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
     return true;
 }
 

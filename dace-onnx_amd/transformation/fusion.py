@@ -17,6 +17,8 @@ MatMul -> Add(tensor of the output's shape)  input connector ``_residual``
 Conv -> Relu                                 ``_activation = "relu"``
 X -> Reshape/Transpose chain -> MatMul       MatMul reads X through ``_a_view`` /
                                              ``_b_view`` (shape, strides)
+MatMul with a constant [K, N] weight         weight copied once as [N, K];
+                                             ``_b_view`` strides [1, K]
 MatMul -> Transpose -> Reshape               MatMul writes the final array through
                                              ``_y_view``
 ===========================================  =====================================
@@ -332,6 +334,51 @@ def _fold_views(sdfg: SDFG, state: SDFGState) -> int:
     return folded
 
 
+def _pretranspose_weights(sdfg: SDFG, state: SDFGState) -> int:
+    """MatMul with a constant 2-D B ([K, N], n-contiguous as ONNX stores it): keep a
+    second copy of the weight laid out [N, K] and let the node read it through a
+    ``_b_view`` of shape [K, N] with strides [1, K]. With both operands contiguous
+    along k every MFMA fragment is a 16-byte LDS / global access (the layout
+    PyTorch's ``nn.Linear`` and ONNX ``Gemm(transB=1)`` use anyway). Done once, at
+    graph-preparation time -- the analogue of the reference's constant folding
+    (``daceml/transformation/constant_folding.py:48``)."""
+    model = getattr(sdfg, "_parent_onnx_model", None)
+    if model is None:
+        return 0
+    from ..onnx.onnx_importer import clean_onnx_name
+    by_clean = {clean_onnx_name(k): k for k in model.weights}
+    done = 0
+    for node in state.nodes():
+        if not _is_op(node, "MatMul") or getattr(node, "_b_view", None) is not None:
+            continue
+        b_e = _in_edge(state, node, "B")
+        if b_e is None or not isinstance(b_e.src, AccessNode) or b_e.src.data not in by_clean:
+            continue
+        if state.in_edges(b_e.src):  # written inside the graph: not a constant
+            continue
+        desc = sdfg.arrays[b_e.src.data]
+        if len(desc.shape) != 2 or not desc.is_contiguous() or desc.dtype.name != "float32":
+            continue
+        k, n = desc.shape
+        if k % 4 or n % 4:
+            continue
+        t_name = b_e.src.data + "_kcontig"
+        if t_name not in sdfg.arrays:
+            sdfg.add_array(t_name, [n, k], desc.dtype, transient=False)
+            model.weights[by_clean[b_e.src.data] + "_kcontig"] = model.weights[by_clean[b_e.src.data]].t().contiguous()
+        t_access = None
+        for cand in state.nodes():
+            if isinstance(cand, AccessNode) and cand.data == t_name:
+                t_access = cand
+        if t_access is None:
+            t_access = state.add_access(t_name)
+        state.remove_edge(b_e)
+        state.add_edge(t_access, None, node, "B", sdfg.make_array_memlet(t_name))
+        node._b_view = ([k, n], [1, k])
+        done += 1
+    return done
+
+
 def _remove_dead_nodes(sdfg: SDFG, state: SDFGState) -> int:
     """Drop nodes whose outputs nobody reads (left behind by the view folds)."""
     removed = 0
@@ -364,6 +411,7 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
     for state in sdfg.nodes():
         total += _fold_into_contractions(sdfg, state)
         total += _fold_views(sdfg, state)
+        total += _pretranspose_weights(sdfg, state)
         _remove_dead_nodes(sdfg, state)
     if total:
         log.info("fused %d patterns in SDFG %s", total, sdfg.name)
