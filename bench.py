@@ -4,8 +4,9 @@
 A step is one BERT-base encoder layer (B=8, S=128, hidden 768, 12 heads, FFN
 3072, fp32) run through ``ONNXModel`` with the "mi355x" expansions: the
 configuration the headline metric is quoted on. Inputs and weights are
-synthetic (seeded) and resident in HBM before the timed region. The launch
-sequence is replayed as one HIP graph per step.
+synthetic (seeded) and resident in HBM before the timed region. A step is
+issued as one HIP-graph replay or as host-issued launches, whichever was
+faster during warm-up (--replay).
 
 Prints one JSON line:
   value / ms_per_step   milliseconds per encoder layer (lower is better)
@@ -106,7 +107,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side oracle timing")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel roofline rows")
-    ap.add_argument("--eager", action="store_true", help="time host-issued launches instead of HIP-graph replay")
+    ap.add_argument("--replay", choices=("auto", "graph", "eager"), default="auto",
+                    help="how a step is issued: one HIP-graph replay, host-issued launches, or (auto) whichever of the "
+                         "two was faster over the warm-up steps")
+    ap.add_argument("--eager", action="store_true", help="same as --replay eager")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB -> 256 MiB elementwise copy three times, so that a counter run of this "
+                         "command holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path has no multi-GPU part (got --gpus {args.gpus}); "
@@ -145,15 +152,31 @@ def main():
     out = torch.empty_like(y)
     call_kwargs = {"x": x, "y": out, **model.clean_weights}
     compiled(**call_kwargs)
-    if args.eager:
-        def step():
-            compiled(**call_kwargs)
+    def eager_step():
+        compiled(**call_kwargs)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / max(n, 1)
+
+    mode = "eager" if args.eager else args.replay
+    if mode == "eager":
+        step = eager_step
     else:
         compiled.capture_graph()
         step = compiled.replay
-
-    for _ in range(args.warmup):
-        step()
+    if mode == "auto":
+        # a graph replay has one launch but a few microseconds between replays; host-issued
+        # launches have none of that but need the host to stay ahead of the GPU
+        timed(eager_step, 5), timed(compiled.replay, 5)
+        t_eager, t_graph = timed(eager_step, args.warmup), timed(compiled.replay, args.warmup)
+        mode, step = ("eager", eager_step) if t_eager < t_graph else ("graph", compiled.replay)
+    else:
+        timed(step, args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -164,6 +187,14 @@ def main():
     torch.cuda.synchronize()
     final_err = float(np.abs(out.cpu().numpy().astype(np.float64) - expected).max() / np.abs(expected).max())
     assert final_err < 1e-4, final_err
+
+    if args.calibrate_copy:
+        src = torch.randn(64 * 1024 * 1024, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- per-kernel durations, HIP events on the launch stream -----------------------------
     kernels = []
@@ -245,7 +276,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "BASELINE config 3: BERT-base encoder layer, B=8 S=128 H=768 heads=12 FFN=3072, "
                                "ONNX graph of MatMul/Add/Reshape/Transpose/Div/Softmax/LayerNormalization/Gelu",
-                   "launches_per_step": compiled.num_launches, "replay": "eager" if args.eager else "hip_graph",
+                   "launches_per_step": compiled.num_launches, "replay": "host_launches" if mode == "eager" else "hip_graph",
                    "max_rel_err_vs_oracle": err},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
     }

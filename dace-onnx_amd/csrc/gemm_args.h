@@ -14,6 +14,7 @@ struct GemmArgs {
     int64_t c_sb0, c_sb1, c_sm;
     int64_t r_sb0, r_sb1, r_sm;
     int64_t tiles_m, tiles_n, nwg;
+    int group_m;  // tile walk order, see tile_coords
     float alpha;
     int epi;
 };

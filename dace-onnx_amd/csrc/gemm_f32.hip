@@ -53,7 +53,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_f32_kernel(GemmAr
     const int64_t tiles_per_batch = p.tiles_m * p.tiles_n;
     const int64_t b = logical / tiles_per_batch, t = logical % tiles_per_batch;
     const int64_t b0 = b / p.batch1, b1 = b % p.batch1;
-    const int64_t m0 = (t / p.tiles_n) * BM, n0 = (t % p.tiles_n) * BN;
+    int64_t tm, tn;
+    tile_coords(t, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const int64_t m0 = tm * BM, n0 = tn * BN;
 
     const float* __restrict__ A = p.A + b0 * p.a_sb0 + b1 * p.a_sb1;
     const float* __restrict__ B = p.B + b0 * p.b_sb0 + b1 * p.b_sb1;
@@ -246,6 +248,10 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     p.tiles_n = ceil_div(N, tc.bn);
     p.nwg = batch * p.tiles_m * p.tiles_n;
     MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "gemm: grid too large (%lld workgroups)", (long long)p.nwg);
+    {   // about two workgroups of these tiles share a CU
+        const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = 2 * (cus / NUM_XCD);
+        p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, tc.bm, tc.bn);
+    }
     launch_config(cfg, p, a_kc, b_kc, vec, static_cast<hipStream_t>(stream));
     return check_launch("gemm_f32_kernel");
 }

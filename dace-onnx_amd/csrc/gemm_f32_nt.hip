@@ -71,7 +71,9 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     const int64_t tiles_per_batch = p.tiles_m * p.tiles_n;
     const int64_t b = logical / tiles_per_batch, t = logical % tiles_per_batch;
     const int64_t b0 = b / p.batch1, b1 = b % p.batch1;
-    const int64_t m0 = (t / p.tiles_n) * BM, n0 = (t % p.tiles_n) * BN;
+    int64_t tm, tn;
+    tile_coords(t, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const int64_t m0 = tm * BM, n0 = tn * BN;
 
     // this lane's A fragment source: row m (clamped into the matrix), 4 floats at
     // k = 32*kt + 16*(c*KSPLIT + ks) + 4*lq for its chunks c
@@ -255,6 +257,10 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     p.tiles_n = ceil_div(p.N, cands[best].bn);
     p.nwg = p.batch * p.tiles_m * p.tiles_n;
     if (p.nwg >= ((int64_t)1 << 31)) return false;
+    // one workgroup per CU at a time: an XCD holds cus / 8 tiles
+    const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD);
+    p.group_m = choose_group_m(p.tiles_m, per_xcd < cus / NUM_XCD ? per_xcd : cus / NUM_XCD, cands[best].bm, cands[best].bn);
+    if (const char* g = getenv("MI355X_GEMM_GROUP_M")) p.group_m = atoi(g) > 0 ? atoi(g) : 1;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
     if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);

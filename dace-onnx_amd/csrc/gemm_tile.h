@@ -18,6 +18,33 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t wg, int64_t nwg) {
     return xcd * full + (xcd < rem ? xcd : rem) + slot;
 }
 
+// Tile t of a tiles_m x tiles_n grid, walked in panels of group_m tile rows, down
+// the panel's rows first. Consecutive t (the slab one XCD works on at a time, see
+// xcd_remap) then cover a group_m x (slab / group_m) block of tiles instead of a
+// single tile row, so the XCD's L2 fetches far fewer distinct operand rows.
+__device__ __forceinline__ void tile_coords(int64_t t, int64_t tiles_m, int64_t tiles_n, int group_m,
+                                            int64_t& tm, int64_t& tn) {
+    const int64_t panel = group_m * tiles_n;
+    const int64_t first_m = (t / panel) * group_m;
+    const int64_t rows = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
+    const int64_t in_panel = t % panel;
+    tm = first_m + in_panel % rows;
+    tn = in_panel / rows;
+}
+
+// Panel height for tile_coords: the block of tiles resident on one XCD at a time
+// (`resident` of them, bm x bn each) should be about square in operand bytes.
+inline int choose_group_m(int64_t tiles_m, int64_t resident, int bm, int bn) {
+    int best = 1;
+    double best_cost = 1e300;
+    for (int g = 1; g <= 16 && g <= tiles_m; ++g) {
+        const double cols = (double)(resident + g - 1) / g;
+        const double cost = g * (double)bm + cols * bn;  // operand rows fetched per k
+        if (cost < best_cost) { best_cost = cost; best = g; }
+    }
+    return best;
+}
+
 // Global -> registers for a ROWS x COLS tile whose COLS direction is the
 // operand's contiguous one. VEC: 16-byte loads (extent along COLS is a multiple
 // of 4 and 16-byte aligned, so a vector is entirely inside or outside).

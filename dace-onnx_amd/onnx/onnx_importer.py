@@ -99,7 +99,9 @@ class ONNXModel:
         self.sdfg._parent_onnx_model = self
         self.cuda = True
         self.state: SDFGState = self.sdfg.add_state()  #: the state containing the model computation
-        self.device = torch.device("cuda:0")
+        # Without a GPU the graph can still be imported, fused and expanded (weights stay
+        # in host memory); compiling or calling it raises.
+        self.device = torch.device("cuda:0" if torch.cuda.is_available() else "cpu")
 
         self.value_infos = {}
         self.inputs: typing.List[str] = []   #: the inputs to the model
@@ -172,6 +174,7 @@ class ONNXModel:
                     self.state.add_edge(op_node, conn_name, access, None, memlet)
 
         self._compiled = None
+        self._expanded = False
         self._static_io = None
 
     # -- construction helpers ----------------------------------------------------------
@@ -223,12 +226,22 @@ class ONNXModel:
         from ..util import utils
         utils.auto_optimize(self.sdfg, cuda=True, fuse=self.fuse)
 
-    def compile_and_init(self):
-        if self._compiled is None:
+    def expand(self):
+        """Apply the graph-level fusion (if enabled) and expand every ONNX node to kernel
+        calls; returns the SDFG. Needs no GPU."""
+        if not self._expanded:
             if self.do_auto_optimize:
                 self.auto_optimize()
             from ..util.utils import expand_onnx_nodes
             expand_onnx_nodes(self.sdfg)
+            self._expanded = True
+        return self.sdfg
+
+    def compile_and_init(self):
+        if self._compiled is None:
+            if self.device.type != "cuda":
+                raise RuntimeError("ONNXModel executes on the MI355X only: no HIP device is visible")
+            self.expand()
             self._compiled = self.sdfg.compile()
         return self._compiled
 

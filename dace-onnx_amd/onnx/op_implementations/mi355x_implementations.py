@@ -127,9 +127,9 @@ class _BatchPlan:
 
 
 def _gemm_call(node, state, plan, a_conn, b_conn, y_conn, bias_conn=None, residual_conn=None,
-               r_strides=None, alpha=1.0, epilogue=_lib.EPI_NONE):
+               r_strides=None, alpha=1.0, epilogue=_lib.EPI_NONE, offsets=(0, 0, 0)):
     return kernel_call_for_node(node, state, "mi355x_gemm_f32", [
-        Ptr(a_conn), Ptr(b_conn), Ptr(y_conn), Ptr(bias_conn), Ptr(residual_conn),
+        Ptr(a_conn, offsets[0]), Ptr(b_conn, offsets[1]), Ptr(y_conn, offsets[2]), Ptr(bias_conn), Ptr(residual_conn),
         plan.batch0, plan.batch1, plan.M, plan.N, plan.K,
         I64Array(plan.a_strides), I64Array(plan.b_strides), I64Array(plan.c_strides),
         I64Array(r_strides) if r_strides is not None else None,
@@ -171,14 +171,20 @@ class MI355XMatMul(ONNXForward):
     @staticmethod
     def _operands(node, state, sdfg):
         """Descriptors of A, B, Y as the kernel will address them: the arrays on the
-        edges, or the (shape, strides) views the fusion pass attached."""
+        edges, or the (shape, strides[, element offset]) views the fusion pass attached."""
         descs = []
         for conn, attr, getter in (("A", "_a_view", in_desc_with_name), ("B", "_b_view", in_desc_with_name),
                                    ("Y", "_y_view", out_desc_with_name)):
             d = getter(node, state, sdfg, conn)
             view = getattr(node, attr, None)
-            descs.append(dace.Array(d.dtype, *view) if view else d)
+            descs.append(dace.Array(d.dtype, view[0], view[1]) if view else d)
         return descs
+
+    @staticmethod
+    def _offsets(node):
+        """Element offsets of the A, B, Y views into the arrays on the edges."""
+        views = [getattr(node, attr, None) for attr in ("_a_view", "_b_view", "_y_view")]
+        return tuple(int(v[2]) if v and len(v) > 2 else 0 for v in views)
 
     @staticmethod
     def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
@@ -197,7 +203,7 @@ class MI355XMatMul(ONNXForward):
             raise ValueError(f"{node.label}: operand layout cannot be expressed as a strided batched GEMM")
         epi, bias_conn, residual_conn, r_strides = _fused_epilogue(node, state, sdfg, plan)
         return _gemm_call(node, state, plan, "A", "B", "Y", bias_conn, residual_conn, r_strides,
-                          alpha=getattr(node, "_alpha", 1.0), epilogue=epi)
+                          alpha=getattr(node, "_alpha", 1.0), epilogue=epi, offsets=MI355XMatMul._offsets(node))
 
 
 @op_implementation(op="Gemm", name=IMPLEMENTATION_NAME)

@@ -245,7 +245,7 @@ class Ptr:
         self.offset = offset        # in elements
 
     def __repr__(self):
-        return f"Ptr({self.connector})"
+        return f"Ptr({self.connector}{'+%d' % self.offset if self.offset else ''})"
 
 
 class Stream:

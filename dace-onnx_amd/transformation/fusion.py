@@ -21,6 +21,10 @@ MatMul with a constant [K, N] weight         weight copied once as [N, K];
                                              ``_b_view`` strides [1, K]
 MatMul -> Transpose -> Reshape               MatMul writes the final array through
                                              ``_y_view``
+MatMuls of one A with constant weights       one MatMul with the weights (and biases)
+(the Q, K, V projections)                    concatenated along N; the readers
+                                             address their slice of the wide result
+                                             through (shape, strides, offset) views
 ===========================================  =====================================
 
 The annotations are private attributes / connectors (leading underscore) that
@@ -271,7 +275,7 @@ def _fold_views(sdfg: SDFG, state: SDFGState) -> int:
 
         def desc_of(edge, view):
             d = sdfg.arrays[edge.data.data]
-            return Array(d.dtype, *view) if view else d
+            return Array(d.dtype, view[0], view[1]) if view else d
 
         views = {"A": getattr(node, "_a_view", None), "B": getattr(node, "_b_view", None),
                  "Y": getattr(node, "_y_view", None)}
@@ -285,8 +289,8 @@ def _fold_views(sdfg: SDFG, state: SDFGState) -> int:
             src_access, shape, strides = found
             trial = dict(views)
             trial[conn] = (shape, strides)
-            plan = _BatchPlan(Array(sdfg.arrays[src_access.data].dtype, *trial["A"]) if trial["A"] else sdfg.arrays[a_e.data.data],
-                              Array(sdfg.arrays[src_access.data].dtype, *trial["B"]) if trial["B"] else sdfg.arrays[b_e.data.data],
+            plan = _BatchPlan(Array(sdfg.arrays[src_access.data].dtype, trial["A"][0], trial["A"][1]) if trial["A"] else sdfg.arrays[a_e.data.data],
+                              Array(sdfg.arrays[src_access.data].dtype, trial["B"][0], trial["B"][1]) if trial["B"] else sdfg.arrays[b_e.data.data],
                               desc_of(y_e, trial["Y"]))
             if not plan.ok:
                 continue
@@ -319,7 +323,7 @@ def _fold_views(sdfg: SDFG, state: SDFGState) -> int:
                     drop.append(use2.dst)
                 if ydesc.is_contiguous() and sdfg.arrays[final_access.data].is_contiguous() and y_strides[-1] == 1:
                     view = (list(ydesc.shape), y_strides)
-                    plan = _BatchPlan(desc_of(a_e, views["A"]), desc_of(b_e, views["B"]), Array(ydesc.dtype, *view))
+                    plan = _BatchPlan(desc_of(a_e, views["A"]), desc_of(b_e, views["B"]), Array(ydesc.dtype, view[0], view[1]))
                     if plan.ok:
                         mids = [y_e.dst] + ([t_access] if final_access is not t_access else [])
                         state.remove_edge(y_e)
@@ -379,6 +383,165 @@ def _pretranspose_weights(sdfg: SDFG, state: SDFGState) -> int:
     return done
 
 
+# ----------------------------------------------------------------------------- horizontal fusion
+def _rebase_strides(shape, strides, n_old, n_new):
+    """A view (shape, strides) into a contiguous [rows, n_old] array, re-expressed
+    for the same elements inside a [rows, n_new] array (n_new >= n_old, same column
+    positions). Dimensions that step whole rows scale by n_new / n_old; dimensions
+    that step inside a row keep their stride. None if a dimension does neither."""
+    out, inside = [], 0
+    for extent, st in zip(shape, strides):
+        if extent == 1 or st == 0:
+            out.append(st)
+        elif st % n_old == 0:
+            out.append(st // n_old * n_new)
+        else:
+            inside += (extent - 1) * st
+            out.append(st)
+    return out if inside < n_old else None
+
+
+def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
+    """MatMul nodes that multiply the same A by different constant [K, N_i] weights
+    (optionally each with a fused 1-D bias) become one MatMul against the weights
+    concatenated along N. Applies when every reader of every Y_i is a MatMul
+    operand, because only the GEMM can address a column slice of the wide result
+    without a copy. One launch instead of len(group), and A is read once."""
+    import torch
+    from ..onnx.onnx_importer import clean_onnx_name
+    from ..onnx.op_implementations.mi355x_implementations import _BatchPlan
+    model = getattr(sdfg, "_parent_onnx_model", None)
+    if model is None:
+        return 0
+    by_clean = {clean_onnx_name(k): k for k in model.weights}
+
+    def constant_input(node, conn, ndim):
+        e = _in_edge(state, node, conn)
+        if e is None or not isinstance(e.src, AccessNode) or e.src.data not in by_clean or state.in_edges(e.src):
+            return None
+        d = sdfg.arrays[e.src.data]
+        if len(d.shape) != ndim or not d.is_contiguous() or d.dtype.name != "float32":
+            return None
+        return e
+
+    groups = {}
+    for node in state.nodes():
+        if not _is_op(node, "MatMul"):
+            continue
+        if any(getattr(node, a, None) is not None for a in ("_a_view", "_b_view", "_y_view", "_activation")) \
+                or getattr(node, "_alpha", 1.0) != 1.0 or _in_edge(state, node, "_residual") is not None:
+            continue
+        a_e, y_e = _in_edge(state, node, "A"), _out_edge(state, node, "Y")
+        b_e = constant_input(node, "B", 2)
+        if a_e is None or b_e is None or y_e is None or not isinstance(a_e.src, AccessNode) \
+                or not isinstance(y_e.dst, AccessNode):
+            continue
+        has_bias = _in_edge(state, node, "_bias") is not None
+        bias_e = constant_input(node, "_bias", 1) if has_bias else None
+        if has_bias and bias_e is None:
+            continue
+        ydesc = sdfg.arrays[y_e.dst.data]
+        if not ydesc.transient or not ydesc.is_contiguous() or len(state.in_edges(y_e.dst)) != 1:
+            continue
+        if any(isinstance(n, AccessNode) and n is not y_e.dst and n.data == y_e.dst.data for n in state.nodes()):
+            continue
+        readers = state.out_edges(y_e.dst)
+        if not readers or not all(_is_op(r.dst, "MatMul") and r.dst_conn in ("A", "B") for r in readers):
+            continue
+        if any(r.dst is node for r in readers):
+            continue
+        k = sdfg.arrays[b_e.src.data].shape[0]
+        a_writes = sum(len(state.in_edges(n)) for n in state.nodes() if isinstance(n, AccessNode) and n.data == a_e.src.data)
+        if a_writes > 1:
+            continue
+        groups.setdefault((a_e.src.data, k, has_bias), []).append((node, a_e, b_e, bias_e, y_e, readers))
+
+    fused = 0
+    for members in groups.values():
+        if len(members) < 2:
+            continue
+        # a reader of one member's output must not be another member (they all run at once)
+        nodes = [m[0] for m in members]
+        if any(r.dst in nodes for m in members for r in m[5]):
+            continue
+        widths = [sdfg.arrays[m[2].src.data].shape[1] for m in members]
+        if any(w % 4 for w in widths):
+            continue
+        n_total = sum(widths)
+        first = members[0]
+        y0 = sdfg.arrays[first[4].dst.data]
+        wide_shape = list(y0.shape[:-1]) + [n_total]
+        if any(list(sdfg.arrays[m[4].dst.data].shape[:-1]) != wide_shape[:-1] for m in members):
+            continue
+        # ---- new views of every reader; give up on the whole group if one cannot be expressed
+        rewires, start, ok = [], 0, True
+        for (node, a_e, b_e, bias_e, y_e, readers), width in zip(members, widths):
+            ydesc = sdfg.arrays[y_e.dst.data]
+            for r in readers:
+                attr = "_a_view" if r.dst_conn == "A" else "_b_view"
+                old = getattr(r.dst, attr, None)
+                shape, strides = (old[0], old[1]) if old else (list(ydesc.shape), list(ydesc.strides))
+                offset = old[2] if old and len(old) > 2 else 0
+                new_strides = _rebase_strides(shape, strides, width, n_total)
+                if new_strides is None or offset != 0:
+                    ok = False
+                    break
+                rewires.append((r, attr, (list(shape), new_strides, start)))
+            start += width
+        if not ok:
+            continue
+        trial = {}
+        for r, attr, view in rewires:
+            trial.setdefault(r.dst, {})[attr] = view
+        for consumer, views in trial.items():
+            def operand(conn, attr):
+                v = views.get(attr, getattr(consumer, attr, None))
+                if v:
+                    return Array(y0.dtype, v[0], v[1])
+                e = _in_edge(state, consumer, conn)
+                return sdfg.arrays[e.data.data]
+            yv = getattr(consumer, "_y_view", None)
+            yd = Array(y0.dtype, yv[0], yv[1]) if yv else sdfg.arrays[_out_edge(state, consumer, "Y").data.data]
+            if not _BatchPlan(operand("A", "_a_view"), operand("B", "_b_view"), yd).ok:
+                ok = False
+        if not ok:
+            continue
+        # ---- constants: weights [K, sum N_i], biases [sum N_i]
+        w_name = by_clean[first[2].src.data] + "_hcat"
+        model.weights[w_name] = torch.cat([model.weights[by_clean[m[2].src.data]] for m in members], dim=1).contiguous()
+        w_clean = clean_onnx_name(w_name)
+        sdfg.add_array(w_clean, list(model.weights[w_name].shape), y0.dtype, transient=False)
+        b_clean = None
+        if first[3] is not None:
+            b_name = by_clean[first[3].src.data] + "_hcat"
+            model.weights[b_name] = torch.cat([model.weights[by_clean[m[3].src.data]].reshape(-1) for m in members]).contiguous()
+            b_clean = clean_onnx_name(b_name)
+            sdfg.add_array(b_clean, [n_total], y0.dtype, transient=False)
+        wide = first[4].dst.data + "_hcat"
+        sdfg.add_transient(wide, wide_shape, y0.dtype)
+        wide_access = state.add_access(wide)
+        # ---- the first member becomes the wide MatMul
+        keep = first[0]
+        state.remove_edge(first[2])
+        state.add_edge(state.add_access(w_clean), None, keep, "B", sdfg.make_array_memlet(w_clean))
+        if b_clean is not None:
+            state.remove_edge(first[3])
+            state.add_edge(state.add_access(b_clean), None, keep, "_bias", sdfg.make_array_memlet(b_clean))
+        state.remove_edge(first[4])
+        state.add_edge(keep, "Y", wide_access, None, sdfg.make_array_memlet(wide))
+        for r, attr, view in rewires:
+            state.remove_edge(r)
+            state.add_edge(wide_access, None, r.dst, r.dst_conn, sdfg.make_array_memlet(wide))
+            setattr(r.dst, attr, view)
+        for node, a_e, b_e, bias_e, y_e, readers in members:
+            if node is not keep:
+                state.remove_node(node)
+            state.remove_node(y_e.dst)
+            del sdfg.arrays[y_e.dst.data]
+        fused += len(members) - 1
+    return fused
+
+
 def _remove_dead_nodes(sdfg: SDFG, state: SDFGState) -> int:
     """Drop nodes whose outputs nobody reads (left behind by the view folds)."""
     removed = 0
@@ -411,6 +574,8 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
     for state in sdfg.nodes():
         total += _fold_into_contractions(sdfg, state)
         total += _fold_views(sdfg, state)
+        _remove_dead_nodes(sdfg, state)  # folded Reshape/Transpose chains must not count as readers
+        total += _fuse_shared_input_matmuls(sdfg, state)
         total += _pretranspose_weights(sdfg, state)
         _remove_dead_nodes(sdfg, state)
     if total:

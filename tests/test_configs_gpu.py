@@ -77,6 +77,31 @@ def test_golden_bert_layer_model(golden, fuse):
     assert np.array_equal(got, got2.cpu().numpy())
 
 
+def test_matmuls_sharing_an_input_are_fused_into_one_wide_gemm():
+    # y1 = x w1 + b1 and y2 = x w2 + b2 become one GEMM; their readers address column slices of its result
+    rng = np.random.default_rng(7)
+    x = rng.normal(size=(3, 20, 32)).astype(np.float32)
+    w1, w2 = rng.normal(size=(32, 24)).astype(np.float32), rng.normal(size=(32, 8)).astype(np.float32)
+    b1, b2 = rng.normal(size=24).astype(np.float32), rng.normal(size=8).astype(np.float32)
+    w3, w4 = rng.normal(size=(24, 12)).astype(np.float32), rng.normal(size=(40, 20)).astype(np.float32)
+    H = proto.helper
+    nodes = [H.make_node("MatMul", ["x", "w1"], ["y1m"]), H.make_node("Add", ["y1m", "b1"], ["y1"]),
+             H.make_node("MatMul", ["x", "w2"], ["y2m"]), H.make_node("Add", ["b2", "y2m"], ["y2"]),
+             H.make_node("MatMul", ["y1", "w3"], ["z1"]), H.make_node("MatMul", ["w4", "y2"], ["z2"])]
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("x", 1, list(x.shape))],
+                     [H.make_tensor_value_info("z1", 1, None), H.make_tensor_value_info("z2", 1, None)],
+                     initializer=[proto.numpy_helper.from_array(a, n) for a, n in
+                                  ((w1, "w1"), (w2, "w2"), (b1, "b1"), (b2, "b2"), (w3, "w3"), (w4, "w4"))])
+    x64 = x.astype(np.float64)
+    want1 = (x64 @ w1 + b1) @ w3
+    want2 = w4.astype(np.float64) @ (x64 @ w2 + b2)
+    for fuse in (False, True):
+        model = donnx.ONNXModel(f"hfuse_{fuse}", H.make_model(g), fuse=fuse)
+        z1, z2 = model(x)
+        assert model.compile_and_init().num_launches == (3 if fuse else 6)
+        assert rel_err(want1, z1) < FP32_REL_TOL and rel_err(want2, z2) < FP32_REL_TOL
+
+
 # ----------------------------------------------------------------------------- config 2: softmax / layernorm
 def test_config2_softmax_full_size():
     X = np.random.default_rng(2).normal(size=(8, 12, 128, 128)).astype(np.float32)

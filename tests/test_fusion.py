@@ -1,0 +1,98 @@
+"""Graph-level fusion pass, checked without a GPU: the model is imported, fused and
+expanded to kernel calls on the host, and the launch list is inspected."""
+import numpy as np
+import pytest
+
+from dace_onnx_amd import sdfg as dace
+import dace_onnx_amd.onnx as donnx
+from dace_onnx_amd.onnx import proto
+from dace_onnx_amd.testing.graphs import bert_encoder_layer_model
+from dace_onnx_amd.transformation.fusion import _rebase_strides, _reshape_strides
+from oracle import pure_ops
+
+H = proto.helper
+
+
+def _launches(model):
+    sdfg = model.expand()
+    out = []
+    for n, _ in sdfg.all_nodes_recursive():
+        if isinstance(n, dace.KernelCall):
+            out.append((n.function, [a.values if isinstance(a, dace.I64Array) else a for a in n.args]))
+    return out
+
+
+def _bert(fuse):
+    w = pure_ops.bert_layer_weights(np.random.default_rng(0), hidden=64, ffn=128)
+    return donnx.ONNXModel("bert_small", bert_encoder_layer_model(w, 2, 16, 4), fuse=fuse)
+
+
+def test_unfused_bert_layer_launches_every_node():
+    names = [f for f, _ in _launches(_bert(False))]
+    assert names.count("mi355x_gemm_f32") == 8 and names.count("mi355x_permute_b32") == 5
+    assert len(names) == 26
+
+
+def test_fused_bert_layer_is_nine_launches():
+    calls = _launches(_bert(True))
+    assert [f for f, _ in calls] == ["mi355x_gemm_f32"] * 2 + ["mi355x_softmax_f32"] + ["mi355x_gemm_f32"] * 2 + \
+        ["mi355x_layernorm_f32"] + ["mi355x_gemm_f32"] * 2 + ["mi355x_layernorm_f32"]
+    qkv, scores, _, ctx, out, _, ffn1, ffn2, _ = [a for _, a in calls]
+    # Q, K, V projections: one GEMM of width 3 * 64 with the concatenated bias, weight k-contiguous
+    assert qkv[5:10] == [1, 1, 32, 192, 64] and qkv[11] == [0, 0, 1, 64] and qkv[15] == 1
+    # Q K^T reads Q at column 0 and K at column 64 of the wide result, scaled by 1/sqrt(16)
+    assert (scores[0].offset, scores[1].offset) == (0, 64)
+    assert scores[5:10] == [2, 4, 16, 16, 16]
+    assert scores[10] == [16 * 192, 16, 192, 1] and scores[11] == [16 * 192, 16, 1, 192]
+    assert scores[14] == pytest.approx(0.25)
+    # P V reads V at column 128 and writes heads merged: [B, S, H * D]
+    assert ctx[1].offset == 128 and ctx[11] == [16 * 192, 16, 192, 1] and ctx[12] == [16 * 64, 16, 64]
+    # output projection and FFN: bias (1), Gelu (4), residual (8) in the epilogue
+    assert out[15] == 9 and ffn1[15] == 5 and ffn2[15] == 9
+
+
+def test_shared_input_matmuls_with_other_readers_are_left_alone():
+    # Y1 is also read by an Add: a column slice of a wide result cannot feed it without a copy
+    rng = np.random.default_rng(1)
+    w1, w2 = rng.normal(size=(8, 12)).astype(np.float32), rng.normal(size=(8, 12)).astype(np.float32)
+    w3 = rng.normal(size=(12, 4)).astype(np.float32)
+    nodes = [H.make_node("MatMul", ["x", "w1"], ["y1"]), H.make_node("MatMul", ["x", "w2"], ["y2"]),
+             H.make_node("MatMul", ["y1", "w3"], ["z1"]), H.make_node("Add", ["y1", "y2"], ["s"])]
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("x", 1, [4, 8])],
+                     [H.make_tensor_value_info("z1", 1, None), H.make_tensor_value_info("s", 1, None)],
+                     initializer=[proto.numpy_helper.from_array(w1, "w1"), proto.numpy_helper.from_array(w2, "w2"),
+                                  proto.numpy_helper.from_array(w3, "w3")])
+    calls = _launches(donnx.ONNXModel("no_hfuse", H.make_model(g)))
+    assert [f for f, _ in calls].count("mi355x_gemm_f32") == 3
+
+
+def test_shared_input_matmuls_read_directly_by_matmuls_are_fused():
+    rng = np.random.default_rng(2)
+    w1, w2 = rng.normal(size=(8, 12)).astype(np.float32), rng.normal(size=(8, 4)).astype(np.float32)
+    w3 = rng.normal(size=(12, 4)).astype(np.float32)
+    nodes = [H.make_node("MatMul", ["x", "w1"], ["y1"]), H.make_node("MatMul", ["x", "w2"], ["y2"]),
+             H.make_node("MatMul", ["y1", "w3"], ["z1"]), H.make_node("MatMul", ["w3", "y2"], ["z2"])]
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("x", 1, [4, 8])],
+                     [H.make_tensor_value_info("z1", 1, None), H.make_tensor_value_info("z2", 1, None)],
+                     initializer=[proto.numpy_helper.from_array(w1, "w1"), proto.numpy_helper.from_array(w2, "w2"),
+                                  proto.numpy_helper.from_array(w3, "w3")])
+    calls = _launches(donnx.ONNXModel("hfuse", H.make_model(g)))
+    assert len(calls) == 3
+    wide, z1, z2 = [a for _, a in calls]
+    assert wide[5:10] == [1, 1, 4, 16, 8]
+    assert z1[0].offset == 0 and z1[10] == [0, 0, 16, 1]      # y1 = columns 0..11 of the [4, 16] result
+    assert z2[1].offset == 12 and z2[11] == [0, 0, 16, 1]     # y2 = columns 12..15, as the B operand
+
+
+def test_rebase_and_reshape_strides():
+    # [B, H, S, D] view of a contiguous [B*S, 768] array, moved into a [B*S, 2304] array
+    assert _rebase_strides([8, 12, 128, 64], [98304, 64, 768, 1], 768, 2304) == [294912, 64, 2304, 1]
+    # a dimension that neither steps whole rows nor stays inside one
+    assert _rebase_strides([4, 100], [100, 1], 64, 128) is None
+    # numpy's no-copy reshape rule
+    assert _reshape_strides([8, 128, 768], [98304, 768, 1], [8, 128, 12, 64]) == [98304, 768, 64, 1]
+    assert _reshape_strides([8, 12, 128, 64], [98304, 64, 768, 1], [8, 12, 8192]) is None
+    a = np.arange(24).reshape(2, 3, 4)
+    v = a.transpose(1, 0, 2)
+    assert _reshape_strides(list(v.shape), [s // 8 for s in v.strides], [3, 8]) is None  # numpy would copy
+    assert _reshape_strides([2, 3, 4], [12, 4, 1], [6, 4]) == [4, 1]
