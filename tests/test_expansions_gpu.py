@@ -271,7 +271,10 @@ def test_reshape_is_a_view_inside_a_graph():
 # ----------------------------------------------------------------------------- MatMulInteger
 @pytest.mark.parametrize("M, N, K, za, zb", [(128, 128, 64, 0, 0), (128, 128, 64, 3, -2), (512, 384, 768, 3, -2),
                                              (100, 52, 37, 5, 7), (130, 260, 48, -128, 127), (1, 1, 1, 1, 1),
-                                             (33, 2, 16, 0, 9), (7, 129, 1000, -7, 0)])
+                                             (33, 2, 16, 0, 9), (7, 129, 1000, -7, 0),
+                                             # K % 128 == 0 and N % 4 == 0: the pipelined kernel, ragged M and N tiles
+                                             (128, 128, 128, 0, 0), (200, 132, 256, 3, -2), (1, 4, 128, -128, 127),
+                                             (257, 388, 640, 0, 11), (129, 124, 1152, -9, 0), (384, 256, 384, 1, 1)])
 def test_matmul_integer_bit_exact(M, N, K, za, zb):
     rng = np.random.default_rng(13)
     A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
