@@ -20,6 +20,8 @@
 #include "gemm_tile.h"
 
 #include <stdlib.h>
+#include <type_traits>
+#include <utility>
 
 namespace mi355x {
 
@@ -51,9 +53,11 @@ struct ConvArgs {
     int OHW;
     FastDiv div_khw, div_kw, div_ohw, div_ow;
     int64_t tiles_m, tiles_p, nwg;
+    int group_m;    // tile walk order, see tile_coords
     int epi;
     int vec_w;      // W tile may use 16-byte loads
     int vec_y;      // Y may use 16-byte stores (OH*OW % 4 == 0, aligned)
+    int x_bytes;    // size of X (gather kernel only; below 2^31)
 };
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool VEC_W>
@@ -191,6 +195,246 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv2d_f32_kernel(Conv
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Kernel for K = C*KH*KW a multiple of 32 (every convolution with C % 32 == 0, and more):
+// the structure of the k-contiguous GEMM kernel (gemm_f32_nt.hip), with the im2col gather
+// as its B loader.
+//   * W [M, K] is k-contiguous: a lane loads its MFMA operand (row oc, 4 consecutive k)
+//     straight from global memory / L2, RING tiles ahead; the 4 wave rows own disjoint
+//     16-row slices of the 64-row tile, nothing is shared, W never touches LDS.
+//   * Xcol is gathered TRANSPOSED: a loader thread owns one output position p and one
+//     k-quad (4 consecutive k = 4 different (c, r, s) taps), reads its 4 input pixels
+//     with 4-byte loads -- lanes run along p, so a wave load covers 64 neighbouring
+//     pixels of one (c, r, s) tap -- and writes them as ONE 16-byte LDS write into a
+//     [p][k] tile. The k-quad of a unit is the same for the whole wave: tap offsets and
+//     pad tests are computed once per wave on the scalar unit. Every MFMA operand read
+//     is then a 16-byte LDS read (the p-contiguous layout of the generic kernel needs
+//     four 4-byte reads per operand, and on this part LDS instructions, not bytes, are
+//     what limits the matrix pipe).
+//   * 8 waves = 4 wave rows x 2 k-split groups (group g multiplies the g-th 16-k chunk
+//     of every 32-k tile, partial sums meet in LDS at the end); three LDS buffers, a
+//     six-deep register ring of gathered pixels, one barrier per tile, the tile's memory
+//     instructions spread between its MFMAs.
+constexpr int CG_BK = 32, CG_THREADS = 512, CG_RING = 6, CG_STAGES = 3, CG_BM = 64;
+constexpr int CG_PITCH = CG_BK + LDS_PAD;
+constexpr int CG_MAX_K = 4608;   // e.g. 512 input channels, 3 x 3
+
+template <int N, class F, int... I>
+__device__ __forceinline__ void cg_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void cg_static_for(F&& f) {
+    cg_static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// TN: 16-position MFMA tiles per wave; BN = 16 TN output positions per workgroup (64 or 128).
+template <int TN>
+__global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs p) {
+    constexpr int BM = CG_BM, BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
+    static_assert(BN % WAVE == 0, "a wave's loader units share their k-quad");
+    constexpr int UNITS = BN * (BK / 4);                 // (position, k-quad) units of one tile
+    static_assert(UNITS % CG_THREADS == 0, "whole units per thread");
+    constexpr int B_PER_T = UNITS / CG_THREADS;
+    constexpr int STAGE = BN * PITCH;
+    constexpr int RED = BM * BN;                         // partial sums of k-split group 1
+    constexpr int LDS_FLOATS = CG_STAGES * STAGE > RED ? CG_STAGES * STAGE : RED;
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    // tap table: for every k = (c, r, s) the element offset of that tap relative to a
+    // position's top-left input pixel (low 27 bits) and the tap index r * KW + s (high 5 bits)
+    __shared__ __attribute__((aligned(16))) uint32_t lds_tap[CG_MAX_K];
+
+    const int tid = threadIdx.x;
+    const int lane = tid % WAVE, wave = tid / WAVE;
+    const int li = lane % 16, lq = lane / 16;
+    const int wm = wave % 4, ks = wave / 4;   // wave row, k-split group
+
+    for (int k = tid; k < p.K; k += CG_THREADS) {
+        const uint32_t c = fdiv((uint32_t)k, p.div_khw);
+        const uint32_t rs = (uint32_t)k - c * (uint32_t)(p.KH * p.KW);
+        const uint32_t r = fdiv(rs, p.div_kw);
+        const uint32_t t = rs - r * (uint32_t)p.KW;
+        lds_tap[k] = (rs << 27) | (c * (uint32_t)(p.H * p.Wd) + r * (uint32_t)(p.dil_h * p.Wd) + t * (uint32_t)p.dil_w);
+    }
+
+    const int64_t logical = xcd_remap(blockIdx.x, p.nwg);
+    int64_t tm, tn;
+    tile_coords(logical, p.tiles_m, p.tiles_p, p.group_m, tm, tn);
+    const int64_t m0 = tm * BM, p0 = tn * BN;
+
+    // W operand of this lane: row oc (clamped), 4 floats at k = 32 kt + 16 ks + 4 lq
+    int64_t am = m0 + 16 * wm + li;
+    am = am < p.M ? am : p.M - 1;
+    const float* __restrict__ a_ptr = p.W + am * p.K + 16 * ks + 4 * lq;
+
+    // loader: this thread's output position (the same for all its units): byte offset of
+    // its top-left input pixel, and one bit per filter tap (r, s) saying whether that tap
+    // falls outside the image (pad) for this position. KH * KW <= 32 is a launch precondition.
+    const int p_local = tid % BN;
+    uint32_t xbase = 0, tap_outside = 0xffffffffu;
+    {
+        const int64_t pp = p0 + p_local;
+        if (pp < p.P) {
+            const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
+            const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
+            const uint32_t oy = fdiv(q, p.div_ow);
+            const uint32_t ox = q - oy * (uint32_t)p.OW;
+            const int iy0 = (int)oy * p.stride_h - p.pad_t;
+            const int ix0 = (int)ox * p.stride_w - p.pad_l;
+            // may point before the image inside the pad: only ever added to tap offsets that bring it back
+            xbase = (uint32_t)(((int)n * p.C * p.H * p.Wd + iy0 * p.Wd + ix0) * 4);
+            tap_outside = 0;
+            for (int r = 0; r < p.KH; ++r)
+                for (int t = 0; t < p.KW; ++t) {
+                    const bool ok = (unsigned)(iy0 + r * p.dil_h) < (unsigned)p.H && (unsigned)(ix0 + t * p.dil_w) < (unsigned)p.Wd;
+                    tap_outside |= (ok ? 0u : 1u) << (r * p.KW + t);
+                }
+        }
+    }
+    // ... and its k-quads: unit it covers k = 32 kt + 4 kq[it] .. + 3, uniform over the wave
+    int kq[B_PER_T], b_lds[B_PER_T];
+#pragma unroll
+    for (int it = 0; it < B_PER_T; ++it) {
+        kq[it] = __builtin_amdgcn_readfirstlane((tid + it * CG_THREADS) / BN);
+        b_lds[it] = p_local * PITCH + 4 * kq[it];
+    }
+
+    f32x4 acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int ktiles = p.K / BK;  // K % 32 == 0 is a launch precondition
+    const int last_tile = ktiles - 1;
+    f32x4 ra[RING];            // W operand of tile t in slot t % RING
+    f32x4 rb[RING][B_PER_T];   // gathered pixels of tile t in slot t % RING
+    f32x4 bf[2][TN];           // X operands of tile t in set t % 2
+
+    auto load_a = [&](f32x4& dst, int kt) __attribute__((always_inline)) {
+        dst = *reinterpret_cast<const f32x4*>(a_ptr + (int64_t)(kt < last_tile ? kt : last_tile) * BK);
+    };
+    auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt) __attribute__((always_inline)) {
+        const int k0 = (kt < last_tile ? kt : last_tile) * BK;
+        // X as a raw buffer: an offset with bit 31 set is out of range and loads 0.0f, so a
+        // padded tap costs no branch and no select (X is smaller than 2 GiB, checked at launch)
+        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.X), 0, p.x_bytes, 0x00020000);
+#pragma unroll
+        for (int it = 0; it < B_PER_T; ++it) {
+            // the four taps of this unit's k-quad: one broadcast read (same address in every lane)
+            const u32x4 taps = *reinterpret_cast<const u32x4*>(lds_tap + k0 + 4 * kq[it]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t off = xbase + ((taps[e] & 0x07ffffffu) << 2);
+                const uint32_t outside = (tap_outside >> (taps[e] >> 27)) & 1u;
+                dst[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(off | (outside << 31)), 0, 0));
+            }
+        }
+    };
+    auto store_b = [&](const f32x4 (&src)[B_PER_T], int stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < B_PER_T; ++it) *reinterpret_cast<f32x4*>(lds + stage * STAGE + b_lds[it]) = src[it];
+    };
+    auto read_b = [&](f32x4 (&dst)[TN], int stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            dst[j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
+    };
+
+    auto tile_step = [&](auto r_tag, int kt) __attribute__((always_inline)) {
+        constexpr int r = decltype(r_tag)::value;
+        constexpr int cur = r & 1;  // RING is even: tile parity == slot parity
+        load_b(rb[r], kt + RING);                           // slot r went to LDS two steps ago
+        load_a(ra[(r + RING - 1) % RING], kt + RING - 1);   // operand consumed in the previous step
+        store_b(rb[(r + 2) % RING], (r + 2) % CG_STAGES);   // tile kt + 2
+        read_b(bf[cur ^ 1], (r + 1) % CG_STAGES);           // tile kt + 1, visible since the last barrier
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[cur][j][s], ra[r][s], acc[j], 0, 0, 0);
+        // Issue order: LDS traffic first (it must have completed at the barrier), then the
+        // gather loads, each memory instruction between MFMAs so that it never queues
+        // behind the other waves' requests while the matrix pipe idles.
+        constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
+        __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
+        __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(DS_RD, 1, 0);
+        }
+#pragma unroll
+        for (int v = 0; v < 4 * B_PER_T + 1; ++v) {
+            __builtin_amdgcn_sched_group_barrier(MFMA, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(VMEM_RD, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(MFMA, 4 * TN, 0);
+        __syncthreads();
+    };
+    static_assert(RING % 2 == 0 && RING % CG_STAGES == 0, "slot index fixes operand set and LDS buffer");
+
+#pragma unroll
+    for (int r = 0; r < RING; ++r) load_a(ra[r], r);  // tiles beyond the last are clamped: no branch
+    __syncthreads();  // tap table complete
+#pragma unroll
+    for (int r = 0; r < RING; ++r) load_b(rb[r], r);
+    store_b(rb[0], 0);
+    store_b(rb[1], 1);
+    __syncthreads();
+    read_b(bf[0], 0);
+
+    // One code path for every tile: near the end of K the look-aheads are clamped to the
+    // last tile, not switched off, so the step body stays branch-free.
+    for (int kt0 = 0; kt0 < ktiles; kt0 += RING) {
+        cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) {
+            const int kt = kt0 + decltype(r_tag)::value;
+            if (kt < ktiles) tile_step(r_tag, kt);  // uniform; only the last group can be partial
+        });
+    }
+
+    // k-split group 1 hands its partial sums to group 0 through LDS
+    {
+        f32x4* red = reinterpret_cast<f32x4*>(lds);
+        if (ks == 1) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) red[(wm * TN + j) * WAVE + lane] = acc[j];
+        }
+        __syncthreads();
+        if (ks == 1) return;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[j] += red[(wm * TN + j) * WAVE + lane];
+    }
+
+    // epilogue: acc[j][r] = Y[oc = m0 + 16 wm + li][p = p0 + 16 j + 4 lq + r]
+    const int64_t oc = m0 + 16 * wm + li;
+    if (oc >= p.M) return;
+    const float bv = (p.epi & MI355X_EPI_BIAS) ? p.bias[oc] : 0.f;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int64_t pp = p0 + 16 * j + 4 * lq;
+        if (pp >= p.P) continue;
+        f32x4 v = acc[j];
+        v.x = apply_epilogue(v.x, p.epi, bv);
+        v.y = apply_epilogue(v.y, p.epi, bv);
+        v.z = apply_epilogue(v.z, p.epi, bv);
+        v.w = apply_epilogue(v.w, p.epi, bv);
+        if (p.vec_y) {
+            const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
+            const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
+            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(p.Y + ((int64_t)n * p.M + oc) * p.OHW + q));
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (pp + r >= p.P) break;
+                const uint32_t n = fdiv((uint32_t)(pp + r), p.div_ohw);
+                const uint32_t q = (uint32_t)(pp + r) - n * (uint32_t)p.OHW;
+                p.Y[((int64_t)n * p.M + oc) * p.OHW + q] = v[r];
+            }
+        }
+    }
+}
+
 template <int BM, int BN, int BK, int WMs, int WNs>
 static void launch_conv(const ConvArgs& p, hipStream_t st) {
     const dim3 grid((unsigned)p.nwg), block(64 * WMs * WNs);
@@ -264,12 +508,35 @@ extern "C" int mi355x_conv2d_f32(const float* X, const float* W, const float* bi
 
     int cus = mi355x_device_cu_count();
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "conv2d: no usable HIP device");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    p.group_m = 1;
+    // K a multiple of the 32-k tile and 16-byte aligned W rows: the gather kernel
+    if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && C * H * Wd < ((int64_t)1 << 27) &&
+        N * C * H * Wd < ((int64_t)1 << 29) && al16(W) && !getenv("MI355X_CONV_CONFIG")) {
+        p.x_bytes = (int)(N * C * H * Wd * 4);
+        // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
+        // at the same rate, so the choice is the number of rounds times the tile width; ties go
+        // to the narrow tile, whose last, partly filled round is shorter
+        auto cost = [&](int bn, int wgs_per_cu) {
+            const int64_t tiles = ceil_div(M, (int64_t)CG_BM) * ceil_div(P, (int64_t)bn);
+            return ceil_div(tiles, (int64_t)cus * wgs_per_cu) * bn * wgs_per_cu;
+        };
+        const bool wide = getenv("MI355X_CONV_GATHER_BN") ? atoi(getenv("MI355X_CONV_GATHER_BN")) == 128
+                                                          : cost(128, 1) < cost(64, 2);
+        const int bn = wide ? 128 : 64;
+        p.tiles_m = ceil_div(M, (int64_t)CG_BM);
+        p.tiles_p = ceil_div(P, (int64_t)bn);
+        p.nwg = p.tiles_m * p.tiles_p;
+        MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "conv2d: grid too large");
+        if (wide) hipLaunchKernelGGL(conv2d_f32_gather_kernel<8>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
+        else hipLaunchKernelGGL(conv2d_f32_gather_kernel<4>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
+        return check_launch("conv2d_f32_gather_kernel");
+    }
     const int cfg = choose_conv_tile(M, P, cus);
     p.tiles_m = ceil_div(M, kConvTiles[cfg].bm);
     p.tiles_p = ceil_div(P, kConvTiles[cfg].bn);
     p.nwg = p.tiles_m * p.tiles_p;
     MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "conv2d: grid too large");
-    hipStream_t st = static_cast<hipStream_t>(stream);
     switch (cfg) {
         case 0: launch_conv<64, 128, 16, 2, 2>(p, st); break;
         case 1: launch_conv<64, 64, 32, 2, 2>(p, st); break;

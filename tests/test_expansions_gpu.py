@@ -119,6 +119,12 @@ def test_conv_config1_stride2():
     ((3, 4, 9, 9), (65, 4, 1, 1), dict(strides=[3, 3])),                       # 1x1 kernel, odd filter count
     ((2, 6, 15, 14), (33, 6, 3, 3), dict(auto_pad="SAME_UPPER", strides=[2, 2])),
     ((1, 2, 30, 31), (4, 2, 5, 3), dict(pads=[2, 1, 2, 1])),                   # OH*OW % 4 != 0: scalar stores
+    # C*KH*KW % 32 == 0: the transposed-gather kernel (64 x 64 and 64 x 128 position tiles, ragged edges)
+    ((2, 32, 12, 12), (64, 32, 3, 3), dict(pads=[1, 1, 1, 1])),
+    ((3, 32, 9, 11), (70, 32, 1, 1), dict()),                                  # K = 32: a single k tile, 70 filters
+    ((2, 8, 14, 13), (5, 8, 2, 2), dict(pads=[0, 1, 1, 0], strides=[2, 1], dilations=[1, 2])),   # odd OH*OW
+    ((40, 16, 30, 30), (48, 16, 3, 2), dict(pads=[2, 0, 1, 3], strides=[1, 2])),                 # many tiles -> 128-wide
+    ((1, 64, 5, 5), (64, 64, 3, 3), dict(auto_pad="SAME_UPPER")),              # K = 576, 25 positions
 ])
 def test_conv_attributes(shape, wshape, attrs):
     rng = np.random.default_rng(4)
