@@ -19,7 +19,7 @@ LIBRARY_PATH = os.path.join(_HERE, LIBRARY_NAME)
 # status codes / flags, mirrored from include/mi355x_onnx.h
 OK = 0
 EPI_NONE, EPI_BIAS, EPI_RELU, EPI_GELU, EPI_RESIDUAL = 0, 1, 2, 4, 8
-OP_ADD, OP_SUB, OP_MUL, OP_DIV = 0, 1, 2, 3
+OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_POW = 0, 1, 2, 3, 4
 OP_RELU, OP_GELU, OP_ERF, OP_SQRT = 16, 17, 18, 19
 
 _c_i64_p = ctypes.POINTER(ctypes.c_int64)
@@ -42,6 +42,7 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
                                         _i64, _i64, _i64, _vp]),
     "mi355x_softmax_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_layernorm_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
+    "mi355x_reduce_mean_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_eltwise_f32": (_int, [_int, _vp, _vp, _vp, _int, _c_i64_p, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_permute_b32": (_int, [_vp, _vp, _int, _c_i64_p, _c_i64_p, _vp]),
 }

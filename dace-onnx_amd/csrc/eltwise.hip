@@ -28,6 +28,7 @@ __device__ __forceinline__ float apply_op(float a, float b) {
     else if constexpr (OP == MI355X_OP_SUB) return a - b;
     else if constexpr (OP == MI355X_OP_MUL) return a * b;
     else if constexpr (OP == MI355X_OP_DIV) return a / b;
+    else if constexpr (OP == MI355X_OP_POW) return b == 2.0f ? a * a : powf(a, b);
     else if constexpr (OP == MI355X_OP_RELU) return fmaxf(a, 0.0f);
     else if constexpr (OP == MI355X_OP_GELU) return gelu_erf(a);
     else if constexpr (OP == MI355X_OP_ERF) return erff(a);
@@ -228,6 +229,7 @@ extern "C" int mi355x_eltwise_f32(int op, const float* A, const float* B, float*
         case MI355X_OP_SUB: return launch_eltwise<MI355X_OP_SUB>(A, B, C, m, st);
         case MI355X_OP_MUL: return launch_eltwise<MI355X_OP_MUL>(A, B, C, m, st);
         case MI355X_OP_DIV: return launch_eltwise<MI355X_OP_DIV>(A, B, C, m, st);
+        case MI355X_OP_POW: return launch_eltwise<MI355X_OP_POW>(A, B, C, m, st);
         case MI355X_OP_RELU: return launch_eltwise<MI355X_OP_RELU>(A, B, C, m, st);
         case MI355X_OP_GELU: return launch_eltwise<MI355X_OP_GELU>(A, B, C, m, st);
         case MI355X_OP_ERF: return launch_eltwise<MI355X_OP_ERF>(A, B, C, m, st);

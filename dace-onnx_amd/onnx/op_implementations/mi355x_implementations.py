@@ -408,6 +408,42 @@ class MI355XSoftmax(ONNXForward):
                                     [Ptr("input"), Ptr("output"), outer, axis_len, inner, Stream()])
 
 
+@op_implementation(op="ReduceMean", name=IMPLEMENTATION_NAME)
+class MI355XReduceMean(ONNXForward):
+    """Mean over ``axes`` (attribute form, opset < 18) when they are adjacent, which
+    makes them one axis of the product length (PureReduceMean, :97-109)."""
+
+    @staticmethod
+    def _split(node, X):
+        """(outer, axis_len, inner, reduced axes) or None."""
+        rank = len(X.shape)
+        axes = sorted(a % rank for a in node.axes) if node.axes is not None else list(range(rank))
+        if not axes or axes != list(range(axes[0], axes[-1] + 1)) or any(not -rank <= a < rank for a in (node.axes or [])):
+            return None
+        return prod(X.shape[:axes[0]]), prod(X.shape[axes[0]:axes[-1] + 1]), prod(X.shape[axes[-1] + 1:]), axes
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "data")
+        Y = out_desc_with_name(node, state, sdfg, "reduced")
+        if not _is_f32(X, Y) or not _contig(X, Y) or len(X.shape) < 1:
+            return False
+        split = MI355XReduceMean._split(node, X)
+        if split is None or split[1] < 1:
+            return False
+        keep = node.keepdims is None or bool(node.keepdims)
+        want = [1 if d in split[3] else e for d, e in enumerate(X.shape)] if keep else \
+            [e for d, e in enumerate(X.shape) if d not in split[3]]
+        return [e for e in Y.shape if e != 1] == [e for e in want if e != 1] and Y.total_size == split[0] * split[2]
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "data")
+        outer, axis_len, inner, _ = MI355XReduceMean._split(node, X)
+        return kernel_call_for_node(node, state, "mi355x_reduce_mean_f32",
+                                    [Ptr("data"), Ptr("reduced"), outer, axis_len, inner, Stream()])
+
+
 @op_implementation(op="LayerNormalization", name=IMPLEMENTATION_NAME)
 class MI355XLayerNormalization(ONNXForward):
     """One-pass layer normalization over the dimensions from ``axis`` on."""
@@ -443,16 +479,18 @@ class MI355XLayerNormalization(ONNXForward):
 # elementwise
 
 
-def _binary_impl(op_name, opcode):
+def _binary_impl(op_name, opcode, conns=("A", "B", "C")):
+    a_conn, b_conn, c_conn = conns
+
     @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
     class Impl(ONNXForward):
-        __doc__ = f"``C = A {op_name.lower()} B`` with numpy broadcasting, one pass."
+        __doc__ = f"``{c_conn} = {a_conn} {op_name.lower()} {b_conn}`` with numpy broadcasting, one pass."
 
         @staticmethod
         def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
-            A = in_desc_with_name(node, state, sdfg, "A")
-            B = in_desc_with_name(node, state, sdfg, "B")
-            C = out_desc_with_name(node, state, sdfg, "C")
+            A = in_desc_with_name(node, state, sdfg, a_conn)
+            B = in_desc_with_name(node, state, sdfg, b_conn)
+            C = out_desc_with_name(node, state, sdfg, c_conn)
             if not _is_f32(A, B, C) or not _contig(C):
                 return False
             out = _broadcast_shape(A.shape, B.shape)
@@ -460,11 +498,11 @@ def _binary_impl(op_name, opcode):
 
         @staticmethod
         def forward(node, state: SDFGState, sdfg: SDFG):
-            A = in_desc_with_name(node, state, sdfg, "A")
-            B = in_desc_with_name(node, state, sdfg, "B")
-            C = out_desc_with_name(node, state, sdfg, "C")
+            A = in_desc_with_name(node, state, sdfg, a_conn)
+            B = in_desc_with_name(node, state, sdfg, b_conn)
+            C = out_desc_with_name(node, state, sdfg, c_conn)
             return kernel_call_for_node(node, state, "mi355x_eltwise_f32", [
-                opcode, Ptr("A"), Ptr("B"), Ptr("C"), len(C.shape), I64Array(C.shape),
+                opcode, Ptr(a_conn), Ptr(b_conn), Ptr(c_conn), len(C.shape), I64Array(C.shape),
                 I64Array(_broadcast_strides(A, C.shape)), I64Array(_broadcast_strides(B, C.shape)), Stream()])
 
     Impl.__name__ = Impl.__qualname__ = "MI355X" + op_name
@@ -475,6 +513,8 @@ MI355XAdd = _binary_impl("Add", _lib.OP_ADD)
 MI355XSub = _binary_impl("Sub", _lib.OP_SUB)
 MI355XMul = _binary_impl("Mul", _lib.OP_MUL)
 MI355XDiv = _binary_impl("Div", _lib.OP_DIV)
+# PurePow (pure_implementations.py:59-74) special-cases the exponent 2 of the exported LayerNorm; so does the kernel
+MI355XPow = _binary_impl("Pow", _lib.OP_POW, conns=("X", "Y", "Z"))
 
 
 def _unary_impl(op_name, opcode, in_conn, out_conn, extra_check=None):

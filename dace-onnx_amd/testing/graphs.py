@@ -13,9 +13,12 @@ import numpy as np
 from ..onnx.proto import helper, numpy_helper, TensorProto
 
 
-def bert_encoder_layer_model(w, batch, seq, heads, eps=1e-12, name="bert_encoder_layer"):
+def bert_encoder_layer_model(w, batch, seq, heads, eps=1e-12, name="bert_encoder_layer", decomposed=False):
     """:param w: dict with wq wk wv wo [H,H], w1 [H,F], w2 [F,H], biases bq bk bv bo b1 b2,
-                 ln1_g ln1_b ln2_g ln2_b (see ``oracle.pure_ops.bert_layer_weights``)."""
+                 ln1_g ln1_b ln2_g ln2_b (see ``oracle.pure_ops.bert_layer_weights``).
+       :param decomposed: write LayerNorm and Gelu the way an opset-12 export does (the form the
+                 reference executes): ReduceMean, Sub, Pow, ReduceMean, Add, Sqrt, Div, Mul, Add and
+                 Div, Erf, Add, Mul, Mul."""
     hidden = w["wq"].shape[0]
     d = hidden // heads
     f32 = TensorProto.FLOAT
@@ -46,17 +49,36 @@ def bert_encoder_layer_model(w, batch, seq, heads, eps=1e-12, name="bert_encoder
     probs = n("Softmax", [scores], "probs", axis=3)
     ctx = n("MatMul", [probs, v], "ctx_heads")
     ctx = n("Reshape", [n("Transpose", [ctx], "ctx_t", perm=[0, 2, 1, 3]), "merge_shape"], "ctx")
+    def layer_norm(x, g, b, out, tag):
+        if not decomposed:
+            return n("LayerNormalization", [x, g, b], out, axis=-1, epsilon=eps)
+        mean = n("ReduceMean", [x], f"{tag}_mean", axes=[-1], keepdims=1)
+        centred = n("Sub", [x, mean], f"{tag}_centred")
+        var = n("ReduceMean", [n("Pow", [centred, "two"], f"{tag}_sq")], f"{tag}_var", axes=[-1], keepdims=1)
+        std = n("Sqrt", [n("Add", [var, "ln_eps"], f"{tag}_var_eps")], f"{tag}_std")
+        normed = n("Div", [centred, std], f"{tag}_normed")
+        return n("Add", [n("Mul", [normed, g], f"{tag}_scaled"), b], out)
+
+    def gelu(x, out):
+        if not decomposed:
+            return n("Gelu", [x], out)
+        t = n("Add", [n("Erf", [n("Div", [x, "sqrt_2"], f"{out}_scaled")], f"{out}_erf"), "one"], f"{out}_erf1")
+        return n("Mul", [n("Mul", [x, t], f"{out}_xerf"), "half"], out)
+
+    if decomposed:
+        inits += [numpy_helper.from_array(np.array(v, dtype=np.float32), k) for k, v in
+                  (("two", 2.0), ("ln_eps", eps), ("sqrt_2", math.sqrt(2.0)), ("one", 1.0), ("half", 0.5))]
     attn = proj(ctx, "wo", "bo", "attn")
-    h1 = n("LayerNormalization", [n("Add", [attn, "x"], "attn_res"), "ln1_g", "ln1_b"], "h1", axis=-1, epsilon=eps)
-    inter = n("Gelu", [proj(h1, "w1", "b1", "ffn1")], "inter")
+    h1 = layer_norm(n("Add", [attn, "x"], "attn_res"), "ln1_g", "ln1_b", "h1", "ln1")
+    inter = gelu(proj(h1, "w1", "b1", "ffn1"), "inter")
     out = proj(inter, "w2", "b2", "ffn2")
-    n("LayerNormalization", [n("Add", [out, h1], "ffn_res"), "ln2_g", "ln2_b"], "y", axis=-1, epsilon=eps)
+    layer_norm(n("Add", [out, h1], "ffn_res"), "ln2_g", "ln2_b", "y", "ln2")
 
     graph = helper.make_graph(nodes, name,
                               [helper.make_tensor_value_info("x", f32, [batch, seq, hidden])],
                               [helper.make_tensor_value_info("y", f32, [batch, seq, hidden])],
                               initializer=inits)
-    return helper.make_model(graph, opset_imports=[helper.make_opsetid("", 17)])
+    return helper.make_model(graph, opset_imports=[helper.make_opsetid("", 12 if decomposed else 17)])
 
 
 def conv_relu_model(W, bias, x_shape, pads=(1, 1, 1, 1), strides=(1, 1), name="conv_relu"):

@@ -21,6 +21,9 @@ MatMul with a constant [K, N] weight         weight copied once as [N, K];
                                              ``_b_view`` strides [1, K]
 MatMul -> Transpose -> Reshape               MatMul writes the final array through
                                              ``_y_view``
+ReduceMean, Sub, Pow(2), ReduceMean,         LayerNormalization (what exporters below
+Add(eps), Sqrt, Div, Mul(gamma), Add(beta)   opset 17 write for ``nn.LayerNorm``)
+Div(sqrt 2), Erf, Add(1), Mul(x), Mul(0.5)   Gelu (exact erf form, any operand order)
 MatMuls of one A with constant weights       one MatMul with the weights (and biases)
 (the Q, K, V projections)                    concatenated along N; the readers
                                              address their slice of the wide result
@@ -383,6 +386,220 @@ def _pretranspose_weights(sdfg: SDFG, state: SDFGState) -> int:
     return done
 
 
+# ----------------------------------------------------------------------------- decomposed operators
+def _other_input(state, node, edge):
+    """The edge into the other operand of a binary node (connectors A and B)."""
+    return _in_edge(state, node, "B" if edge.dst_conn == "A" else "A")
+
+
+def _scalar_constant(sdfg, edge) -> typing.Optional[float]:
+    if edge is None or not isinstance(edge.src, AccessNode):
+        return None
+    val = _constant_value(sdfg, edge.src.data)
+    return float(val.reshape(-1)[0]) if val is not None and val.size == 1 else None
+
+
+def _next_op(sdfg, state, access, *ops):
+    """The single reader of ``access`` if it is one of ``ops`` and ``access`` is a
+    transient written once; else None."""
+    use = _single_consumer(sdfg, state, access)
+    return use if use is not None and _is_op(use.dst, *ops) else None
+
+
+def _out_access(state, node, conn):
+    e = _out_edge(state, node, conn)
+    return e.dst if e is not None and isinstance(e.dst, AccessNode) else None
+
+
+def _drop_chain(sdfg, state, nodes, keep_access):
+    """Remove ``nodes`` and the transients only they touched (never ``keep_access``)."""
+    touched = []
+    for n in nodes:
+        for e in state.in_edges(n) + state.out_edges(n):
+            a = e.src if e.dst is n else e.dst
+            if isinstance(a, AccessNode) and a not in touched:
+                touched.append(a)
+        state.remove_node(n)
+    for a in touched:
+        if a in keep_access:
+            continue
+        if not state.in_edges(a) and not state.out_edges(a):
+            state.remove_node(a)
+            desc = sdfg.arrays.get(a.data)
+            still_used = any(isinstance(n, AccessNode) and n.data == a.data for n in state.nodes())
+            if desc is not None and desc.transient and not still_used:
+                del sdfg.arrays[a.data]
+
+
+def _fuse_decomposed_layernorm(sdfg: SDFG, state: SDFGState) -> int:
+    """ReduceMean(x) -> Sub(x, mean) -> Pow(.,2) -> ReduceMean -> Add(eps) -> Sqrt ->
+    Div(centred, std) -> Mul(gamma) [-> Add(beta)], over the last axis, becomes one
+    LayerNormalization node. This is the decomposition the reference executes node
+    by node (pure_implementations.py:97-109, 82-84, 59-74, 77-79, 41-56, 92-94)."""
+    from ..onnx.nodes.onnx_op import get_onnx_node
+    fused = 0
+    for m1 in list(state.nodes()):
+        if m1 not in state.nodes() or not _is_op(m1, "ReduceMean"):
+            continue
+        x_e = _in_edge(state, m1, "data")
+        mean = _out_access(state, m1, "reduced")
+        if x_e is None or mean is None or not isinstance(x_e.src, AccessNode):
+            continue
+        xdesc = sdfg.arrays[x_e.src.data]
+        rank = len(xdesc.shape)
+        last_axis = lambda n: n.axes is not None and [a % rank for a in n.axes] == [rank - 1] and \
+            (n.keepdims is None or bool(n.keepdims))
+        if rank < 1 or not last_axis(m1) or not xdesc.is_contiguous():
+            continue
+        sub_use = _next_op(sdfg, state, mean, "Sub")
+        if sub_use is None or sub_use.dst_conn != "B":
+            continue
+        sub = sub_use.dst
+        if _in_edge(state, sub, "A").src.data != x_e.src.data:
+            continue
+        centred = _out_access(state, sub, "C")
+        if centred is None or not sdfg.arrays[centred.data].transient or len(state.in_edges(centred)) != 1:
+            continue
+        readers = state.out_edges(centred)
+        pow_e = [e for e in readers if _is_op(e.dst, "Pow") and e.dst_conn == "X"]
+        div_e = [e for e in readers if _is_op(e.dst, "Div") and e.dst_conn == "A"]
+        if len(readers) != 2 or len(pow_e) != 1 or len(div_e) != 1:
+            continue
+        pw, div = pow_e[0].dst, div_e[0].dst
+        if _scalar_constant(sdfg, _in_edge(state, pw, "Y")) != 2.0:
+            continue
+        sq = _out_access(state, pw, "Z")
+        m2_use = _next_op(sdfg, state, sq, "ReduceMean") if sq is not None else None
+        if m2_use is None or not last_axis(m2_use.dst):
+            continue
+        m2 = m2_use.dst
+        var = _out_access(state, m2, "reduced")
+        add_use = _next_op(sdfg, state, var, "Add") if var is not None else None
+        if add_use is None:
+            continue
+        add_eps = add_use.dst
+        eps = _scalar_constant(sdfg, _other_input(state, add_eps, add_use))
+        var_eps = _out_access(state, add_eps, "C")
+        sqrt_use = _next_op(sdfg, state, var_eps, "Sqrt") if var_eps is not None and eps is not None else None
+        if sqrt_use is None:
+            continue
+        sqrt = sqrt_use.dst
+        std = _out_access(state, sqrt, "Y")
+        std_use = _next_op(sdfg, state, std, "Div") if std is not None else None
+        if std_use is None or std_use.dst is not div or std_use.dst_conn != "B":
+            continue
+        normed = _out_access(state, div, "C")
+        mul_use = _next_op(sdfg, state, normed, "Mul") if normed is not None else None
+        if mul_use is None:
+            continue
+        mul = mul_use.dst
+        gamma_e = _other_input(state, mul, mul_use)
+        cols = xdesc.shape[-1]
+
+        def is_row_vector(e):
+            if e is None or not isinstance(e.src, AccessNode):
+                return False
+            d = sdfg.arrays[e.src.data]
+            return d.total_size == cols and d.shape and d.shape[-1] == cols and d.is_contiguous()
+
+        if not is_row_vector(gamma_e):
+            continue
+        out = _out_access(state, mul, "C")
+        if out is None or tuple(sdfg.arrays[out.data].shape) != tuple(xdesc.shape):
+            continue
+        chain = [m1, sub, pw, m2, add_eps, sqrt, div, mul]
+        beta_e = None
+        add_use2 = _next_op(sdfg, state, out, "Add")
+        if add_use2 is not None and is_row_vector(_other_input(state, add_use2.dst, add_use2)):
+            out2 = _out_access(state, add_use2.dst, "C")
+            if out2 is not None and tuple(sdfg.arrays[out2.data].shape) == tuple(xdesc.shape):
+                beta_e = _other_input(state, add_use2.dst, add_use2)
+                chain.append(add_use2.dst)
+                out = out2
+        if not sdfg.arrays[out.data].is_contiguous():
+            continue
+        ln = get_onnx_node("LayerNormalization")(m1.label + "_layernorm", axis=-1, epsilon=eps)
+        state.add_node(ln)
+        ln.add_in_connector("X")
+        state.add_edge(x_e.src, None, ln, "X", sdfg.make_array_memlet(x_e.src.data))
+        ln.add_in_connector("Scale")
+        state.add_edge(gamma_e.src, None, ln, "Scale", sdfg.make_array_memlet(gamma_e.src.data))
+        if beta_e is not None:
+            ln.add_in_connector("B")
+            state.add_edge(beta_e.src, None, ln, "B", sdfg.make_array_memlet(beta_e.src.data))
+        ln.add_out_connector("Y")
+        keep = [x_e.src, gamma_e.src, out] + ([beta_e.src] if beta_e is not None else [])
+        _drop_chain(sdfg, state, chain, keep)
+        state.add_edge(ln, "Y", out, None, sdfg.make_array_memlet(out.data))
+        fused += 1
+    return fused
+
+
+def _fuse_decomposed_gelu(sdfg: SDFG, state: SDFGState) -> int:
+    """x / sqrt(2) (or x * 1/sqrt(2)) -> Erf -> + 1 -> * x -> * 0.5, with the last two
+    multiplications in either order, becomes one Gelu node."""
+    from ..onnx.nodes.onnx_op import get_onnx_node
+    fused = 0
+    for erf in list(state.nodes()):
+        if erf not in state.nodes() or not _is_op(erf, "Erf"):
+            continue
+        scaled_e = _in_edge(state, erf, "input")
+        if scaled_e is None or not isinstance(scaled_e.src, AccessNode) or _single_consumer(sdfg, state, scaled_e.src) is None:
+            continue
+        prod_e = _producer(state, scaled_e.src)
+        if prod_e is None or not _is_op(prod_e.src, "Div", "Mul"):
+            continue
+        scale = prod_e.src
+        a_e, b_e = _in_edge(state, scale, "A"), _in_edge(state, scale, "B")
+        if _is_op(scale, "Div"):
+            x_e, c = a_e, _scalar_constant(sdfg, b_e)
+            ok = c is not None and abs(c - 2.0 ** 0.5) < 1e-4
+        else:
+            ca, cb = _scalar_constant(sdfg, a_e), _scalar_constant(sdfg, b_e)
+            x_e, c = (b_e, ca) if ca is not None else (a_e, cb)
+            ok = c is not None and abs(c - 0.5 ** 0.5) < 1e-4
+        if not ok or x_e is None or not isinstance(x_e.src, AccessNode):
+            continue
+        x_name = x_e.src.data
+        erf_out = _out_access(state, erf, "output")
+        add_use = _next_op(sdfg, state, erf_out, "Add") if erf_out is not None else None
+        if add_use is None or _scalar_constant(sdfg, _other_input(state, add_use.dst, add_use)) != 1.0:
+            continue
+        add1 = add_use.dst
+        cur = _out_access(state, add1, "C")
+        chain, seen_x, seen_half = [scale, erf, add1], False, False
+        for _ in range(2):  # the two multiplications, either order
+            mul_use = _next_op(sdfg, state, cur, "Mul") if cur is not None else None
+            if mul_use is None:
+                break
+            other = _other_input(state, mul_use.dst, mul_use)
+            if other is None or not isinstance(other.src, AccessNode):
+                break
+            if not seen_x and other.src.data == x_name:
+                seen_x = True
+            elif not seen_half and _scalar_constant(sdfg, other) == 0.5:
+                seen_half = True
+            else:
+                break
+            chain.append(mul_use.dst)
+            cur = _out_access(state, mul_use.dst, "C")
+        # 0.5 may also have been applied to x before the product: x * 0.5 * (1 + erf) is not matched here
+        if not (seen_x and seen_half) or cur is None:
+            continue
+        xdesc, ydesc = sdfg.arrays[x_name], sdfg.arrays[cur.data]
+        if tuple(xdesc.shape) != tuple(ydesc.shape) or not xdesc.is_contiguous() or not ydesc.is_contiguous():
+            continue
+        gelu = get_onnx_node("Gelu")(erf.label + "_gelu")
+        state.add_node(gelu)
+        gelu.add_in_connector("X")
+        state.add_edge(x_e.src, None, gelu, "X", sdfg.make_array_memlet(x_name))
+        gelu.add_out_connector("Y")
+        _drop_chain(sdfg, state, chain, [x_e.src, cur])
+        state.add_edge(gelu, "Y", cur, None, sdfg.make_array_memlet(cur.data))
+        fused += 1
+    return fused
+
+
 # ----------------------------------------------------------------------------- horizontal fusion
 def _rebase_strides(shape, strides, n_old, n_new):
     """A view (shape, strides) into a contiguous [rows, n_old] array, re-expressed
@@ -572,6 +789,8 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
     """Apply every fusion pattern to every state; returns the number of folds."""
     total = 0
     for state in sdfg.nodes():
+        total += _fuse_decomposed_layernorm(sdfg, state)
+        total += _fuse_decomposed_gelu(sdfg, state)
         total += _fold_into_contractions(sdfg, state)
         total += _fold_views(sdfg, state)
         _remove_dead_nodes(sdfg, state)  # folded Reshape/Transpose chains must not count as readers

@@ -136,10 +136,21 @@ int mi355x_layernorm_f32(const float* X, const float* gamma, const float* beta,
                          float* Y, int64_t rows, int64_t cols, float eps,
                          void* stream);
 
+/* ONNX ReduceMean along one axis, fp32. X viewed as [outer, axis_len, inner]
+ * (C-contiguous); Y is [outer, inner] (keepdims only changes the shape the
+ * caller gives it). Replaces PureReduceMean.forward
+ * (pure_implementations.py:97-109), which the reference meets in every
+ * exported LayerNorm (opset 12 has no LayerNormalization node). Several
+ * adjacent reduced axes are one axis of the product length. */
+int mi355x_reduce_mean_f32(const float* X, float* Y,
+                           int64_t outer, int64_t axis_len, int64_t inner,
+                           void* stream);
+
 /* Elementwise ops, fp32, with numpy broadcasting.
  * Replaces the one-map expansions Add/Sub/Mul/Div
- * (pure_implementations.py:77-94), PureRelu (:462-474), PureErf (:112-127),
- * PureSqrt (:41-56) and the Gelu decomposition Div,Erf,Add,Mul,Mul.
+ * (pure_implementations.py:77-94), PurePow (:59-74), PureRelu (:462-474),
+ * PureErf (:112-127), PureSqrt (:41-56) and the Gelu decomposition
+ * Div,Erf,Add,Mul,Mul.
  *   binary ops: C = A op B; unary ops ignore B (pass NULL).
  *   ndim <= 8; shape is the OUTPUT shape; a_strides / b_strides are element
  *   strides of each operand in the output's index space (0 on broadcast dims).
@@ -148,6 +159,7 @@ int mi355x_layernorm_f32(const float* X, const float* gamma, const float* beta,
 #define MI355X_OP_SUB 1
 #define MI355X_OP_MUL 2
 #define MI355X_OP_DIV 3
+#define MI355X_OP_POW 4
 #define MI355X_OP_RELU 16
 #define MI355X_OP_GELU 17
 #define MI355X_OP_ERF 18

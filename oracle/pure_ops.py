@@ -242,6 +242,11 @@ def sqrt(X):
     return np.sqrt(X)
 
 
+def pow(X, Y):  # noqa: A001 (named after the ONNX op)
+    """PurePow (pure_implementations.py:59-74): x ** y, with broadcasting."""
+    return np.power(X, np.asarray(Y, dtype=X.dtype)).astype(X.dtype, copy=False)
+
+
 def transpose(X, perm=None):
     """PureTranspose (pure_implementations.py:369-379)."""
     return np.ascontiguousarray(np.transpose(X, axes=perm))

@@ -236,6 +236,28 @@ def test_unary_ops(shape):
     assert rel_err(O.sqrt(np.abs(X)), Y) < 1e-6
 
 
+@pytest.mark.parametrize("shape, axes, keepdims", [((8, 16, 768), [-1], 1), ((5, 33), [1], 0), ((4, 6, 10), [1], 1),
+                                                   ((3, 4, 5, 6), [1, 2], 0), ((7, 9), [0, 1], 1), ((2, 4100), [-1], 1)])
+def test_reduce_mean(shape, axes, keepdims):
+    X = np.random.default_rng(15).normal(1.0, 2.0, size=shape).astype(np.float32)
+    expected = O.reduce_mean(X.astype(np.float64), axes, keepdims)
+    Y = np.zeros(expected.shape, np.float32)
+    donnx.ONNXReduceMean(data=X, reduced=Y, axes=axes, keepdims=keepdims)
+    assert rel_err(expected, Y) < FP32_REL_TOL
+
+
+def test_pow():
+    rng = np.random.default_rng(16)
+    X = rng.normal(size=(8, 16, 64)).astype(np.float32)
+    Z = np.zeros_like(X)
+    donnx.ONNXPow(X=X, Y=np.array(2.0, np.float32), Z=Z)
+    assert np.array_equal(O.pow(X, 2.0), Z)                 # the exponent of the exported LayerNorm: exact
+    P = np.abs(X) + 0.25
+    E = rng.uniform(-2, 3, size=(64, )).astype(np.float32)  # broadcast exponent
+    donnx.ONNXPow(X=P, Y=E, Z=Z)
+    assert rel_err(O.pow(P.astype(np.float64), E.astype(np.float64)), Z) < FP32_REL_TOL
+
+
 # ----------------------------------------------------------------------------- data movement
 @pytest.mark.parametrize("shape, perm", [((8, 16, 12, 64), (0, 2, 1, 3)), ((2, 12, 16, 64), (0, 1, 3, 2)),
                                          ((5, 7), None), ((3, 4, 5), (2, 0, 1)), ((70, 130), (1, 0)), ((6, ), (0, ))])

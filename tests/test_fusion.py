@@ -84,6 +84,62 @@ def test_shared_input_matmuls_read_directly_by_matmuls_are_fused():
     assert z2[1].offset == 12 and z2[11] == [0, 0, 16, 1]     # y2 = columns 12..15, as the B operand
 
 
+def test_decomposed_layernorm_and_gelu_are_recognised():
+    # the opset-12 export form the reference executes node by node: 46 launches as written, 9 fused
+    w = pure_ops.bert_layer_weights(np.random.default_rng(0), hidden=64, ffn=128)
+    plain = [f for f, _ in _launches(donnx.ONNXModel("d0", bert_encoder_layer_model(w, 2, 16, 4, decomposed=True), fuse=False))]
+    assert len(plain) == 46 and plain.count("mi355x_reduce_mean_f32") == 4
+    fused = _launches(donnx.ONNXModel("d1", bert_encoder_layer_model(w, 2, 16, 4, decomposed=True)))
+    names = [f for f, _ in fused]
+    assert len(names) == 9 and names.count("mi355x_layernorm_f32") == 2 and names.count("mi355x_gemm_f32") == 6
+    ln = [a for f, a in fused if f == "mi355x_layernorm_f32"][0]
+    assert ln[4:6] == [32, 64] and ln[6] == pytest.approx(1e-12)
+    assert sorted(a[15] for f, a in fused if f == "mi355x_gemm_f32") == [0, 0, 1, 5, 9, 9]   # Gelu folded into FFN1
+
+
+def _chain_model(nodes, consts, shape=(4, 8)):
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("x", 1, list(shape))],
+                     [H.make_tensor_value_info("y", 1, None)],
+                     initializer=[proto.numpy_helper.from_array(np.array(v, dtype=np.float32), k) for k, v in consts.items()])
+    return H.make_model(g)
+
+
+def test_gelu_pattern_variants():
+    consts = {"r2": 2.0 ** 0.5, "ir2": 0.5 ** 0.5, "one": 1.0, "half": 0.5}
+    mk = H.make_node
+    variants = {
+        "div, (x * t) * 0.5": [mk("Div", ["x", "r2"], ["s"]), mk("Erf", ["s"], ["e"]), mk("Add", ["e", "one"], ["t"]),
+                               mk("Mul", ["x", "t"], ["u"]), mk("Mul", ["u", "half"], ["y"])],
+        "mul by 1/sqrt2, (t * 0.5) * x": [mk("Mul", ["ir2", "x"], ["s"]), mk("Erf", ["s"], ["e"]), mk("Add", ["one", "e"], ["t"]),
+                                          mk("Mul", ["half", "t"], ["u"]), mk("Mul", ["u", "x"], ["y"])],
+    }
+    for label, nodes in variants.items():
+        calls = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))
+        assert [(f, a[0]) for f, a in calls] == [("mi355x_eltwise_f32", 17)], label
+    # a different constant is not Gelu: the five nodes stay
+    bad = dict(consts, r2=1.5)
+    assert len(_launches(donnx.ONNXModel("g", _chain_model(variants["div, (x * t) * 0.5"], bad)))) == 5
+    # erf(x / sqrt 2) with another reader of the intermediate stays too
+    nodes = variants["div, (x * t) * 0.5"][:-1] + [mk("Mul", ["u", "e"], ["y"])]
+    assert len(_launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))) == 5
+
+
+def test_layernorm_pattern_needs_the_exact_chain():
+    mk = H.make_node
+    consts = {"two": 2.0, "three": 3.0, "eps": 1e-5, "g": np.ones(8), "b": np.zeros(8)}
+
+    def chain(exponent="two", axes=(-1, )):
+        return [mk("ReduceMean", ["x"], ["m"], axes=list(axes), keepdims=1), mk("Sub", ["x", "m"], ["c"]),
+                mk("Pow", ["c", exponent], ["p"]), mk("ReduceMean", ["p"], ["v"], axes=list(axes), keepdims=1),
+                mk("Add", ["v", "eps"], ["ve"]), mk("Sqrt", ["ve"], ["s"]), mk("Div", ["c", "s"], ["n"]),
+                mk("Mul", ["n", "g"], ["sc"]), mk("Add", ["sc", "b"], ["y"])]
+
+    calls = _launches(donnx.ONNXModel("ln", _chain_model(chain(), consts)))
+    assert [f for f, _ in calls] == ["mi355x_layernorm_f32"] and calls[0][1][6] == pytest.approx(1e-5)
+    assert len(_launches(donnx.ONNXModel("ln3", _chain_model(chain(exponent="three"), consts)))) == 9
+    assert len(_launches(donnx.ONNXModel("ln0", _chain_model(chain(axes=(0, )), dict(consts, g=np.ones(8)))))) == 9
+
+
 def test_rebase_and_reshape_strides():
     # [B, H, S, D] view of a contiguous [B*S, 768] array, moved into a [B*S, 2304] array
     assert _rebase_strides([8, 12, 128, 64], [98304, 64, 768, 1], 768, 2304) == [294912, 64, 2304, 1]

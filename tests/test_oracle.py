@@ -194,6 +194,21 @@ def test_gelu_erf_relu_closed_forms():
     assert O.relu(x).dtype == np.float32
 
 
+def test_pow_and_reduce_mean_closed_forms():
+    rng = np.random.default_rng(21)
+    x = rng.normal(size=(3, 5, 7)).astype(np.float32)
+    assert np.array_equal(O.pow(x, 2.0), x * x)                                    # the exponent of the exported LayerNorm
+    pos = np.abs(x) + 0.5
+    ref = np.array([math.pow(float(v), 1.5) for v in pos.reshape(-1)]).reshape(pos.shape)
+    assert rel_err(ref, O.pow(pos, np.float32(1.5))) < TOL
+    m = O.reduce_mean(x, [-1])
+    assert m.shape == (3, 5, 1) and m.dtype == np.float32
+    brute = np.array([[sum(float(v) for v in x[i, j]) / 7 for j in range(5)] for i in range(3)])
+    assert rel_err(brute, m[..., 0]) < TOL
+    assert O.reduce_mean(x, [1, 2], keepdims=0).shape == (3, ) and O.reduce_mean(x, [0], keepdims=1).shape == (1, 5, 7)
+    assert np.allclose(O.reduce_mean(np.full((4, 6), 2.5, np.float32), [1]), 2.5)
+
+
 def test_add_broadcasting():
     rng = np.random.default_rng(9)
     a = rng.normal(size=(8, 16, 24)).astype(np.float32)
