@@ -66,6 +66,9 @@ def algorithmic_work(name, args):
         flops = 2.0 * b0 * b1 * M * N * K
         nbytes = 4.0 * b0 * b1 * (M * K + K * N + M * N * (2 if epi & 8 else 1))
         return flops, nbytes
+    if name == "mi355x_attention_f32":
+        b0, b1, sq, sk, d = args[4:9]
+        return 4.0 * b0 * b1 * sq * sk * d, 4.0 * b0 * b1 * (2 * sq * d + 2 * sk * d)
     if name == "mi355x_softmax_f32":
         outer, n, inner = args[2:5]
         return 0.0, 8.0 * outer * n * inner
@@ -210,6 +213,9 @@ def main():
                 gemm_us += us
                 label = "gemm_f32 b{}x{} {}x{}x{} epi={}".format(*plain[5:10], plain[15])
                 kernels.append(kernel_row(label, us, flops, nbytes, "mfma"))
+            elif name == "mi355x_attention_f32":
+                label = "attention_f32 b{}x{} q{} k{} d{}".format(*plain[4:9])
+                kernels.append(kernel_row(label, us, flops, nbytes, "mfma"))
             else:
                 label = name.replace("mi355x_", "") + " " + "x".join(str(v) for v in (plain[5] if name == "mi355x_eltwise_f32"
                                                                                      else plain[3] if name == "mi355x_permute_b32"
@@ -252,7 +258,8 @@ def main():
         achieved = gemm_flops / gemm_us / 1e6
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
-                    "kernel": "gemm_f32_kernel (all GEMM launches of one layer)",
+                    "kernel": "gemm_f32_nt_kernel (all mi355x_gemm_f32 launches of one layer: QKV, output projection, FFN1, "
+                              "FFN2; the attention core runs in its own fused kernel, listed under kernels)",
                     "flop_per_layer": gemm_flops, "us_per_layer": round(gemm_us, 2)}
 
     # ---- CPU baseline: the oracle's layer on this box's host cores ---------------------------

@@ -408,6 +408,64 @@ class MI355XSoftmax(ONNXForward):
                                     [Ptr("input"), Ptr("output"), outer, axis_len, inner, Stream()])
 
 
+@op_implementation(op="FusedAttention", name=IMPLEMENTATION_NAME)
+class MI355XFusedAttention(ONNXForward):
+    """``softmax(scale * Q K^T) V`` in one launch; scores stay in registers. The
+    operands are the arrays on the edges or the (shape, strides, offset) views the
+    fusion pass attached (``_q_view`` ... ``_o_view``): head split / merge of a
+    [B, S, H*D] projection is addressing, not a copy."""
+
+    SUPPORTED_KEYS, SUPPORTED_HEAD = 128, 64
+
+    @staticmethod
+    def _operands(node, state, sdfg):
+        out = []
+        for conn, attr, getter in (("Q", "_q_view", in_desc_with_name), ("K", "_k_view", in_desc_with_name),
+                                   ("V", "_v_view", in_desc_with_name), ("O", "_o_view", out_desc_with_name)):
+            d = getter(node, state, sdfg, conn)
+            view = getattr(node, attr, None)
+            out.append((dace.Array(d.dtype, view[0], view[1]) if view else d, int(view[2]) if view and len(view) > 2 else 0))
+        return out
+
+    @staticmethod
+    def _plan(descs):
+        """(batch0, batch1, Sq, Sk, D, [strides of Q, K, V, O as {b0, b1, row}]) or None."""
+        (Q, _), (K, _), (V, _), (O, _) = descs
+        if not _is_f32(Q, K, V, O) or min(len(d.shape) for d in (Q, K, V, O)) < 2:
+            return None
+        batch = tuple(Q.shape[:-2])
+        if any(tuple(d.shape[:-2]) != batch for d in (K, V, O)) or len([e for e in batch if e != 1]) > 2:
+            return None
+        (Sq, D), (Sk, D2) = Q.shape[-2:], K.shape[-2:]
+        if D2 != D or tuple(V.shape[-2:]) != (Sk, D) or tuple(O.shape[-2:]) != (Sq, D):
+            return None
+        if any(d.strides[-1] != 1 for d in (Q, K, V, O)):
+            return None
+        if any(st % 4 or st < 0 for d in (Q, K, V, O) for st, e in zip(d.strides[:-1], d.shape[:-1]) if e != 1):
+            return None
+        dims = [i for i, e in enumerate(batch) if e != 1]
+        dims = [None] * (2 - len(dims)) + dims
+        ext = [1 if i is None else batch[i] for i in dims]
+        strides = [[0 if i is None else d.strides[i] for i in dims] + [d.strides[-2]] for d in (Q, K, V, O)]
+        return ext[0], ext[1], Sq, Sk, D, strides
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        plan = MI355XFusedAttention._plan(MI355XFusedAttention._operands(node, state, sdfg))
+        return plan is not None and plan[3] == MI355XFusedAttention.SUPPORTED_KEYS and \
+            plan[4] == MI355XFusedAttention.SUPPORTED_HEAD
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        descs = MI355XFusedAttention._operands(node, state, sdfg)
+        b0, b1, Sq, Sk, D, strides = MI355XFusedAttention._plan(descs)
+        offs = [o for _, o in descs]
+        return kernel_call_for_node(node, state, "mi355x_attention_f32", [
+            Ptr("Q", offs[0]), Ptr("K", offs[1]), Ptr("V", offs[2]), Ptr("O", offs[3]), b0, b1, Sq, Sk, D,
+            I64Array(strides[0]), I64Array(strides[1]), I64Array(strides[2]), I64Array(strides[3]),
+            float(node.scale if node.scale is not None else 1.0), Stream()])
+
+
 @op_implementation(op="ReduceMean", name=IMPLEMENTATION_NAME)
 class MI355XReduceMean(ONNXForward):
     """Mean over ``axes`` (attribute form, opset < 18) when they are adjacent, which

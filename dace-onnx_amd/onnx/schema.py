@@ -132,6 +132,11 @@ SCHEMAS: typing.List[ONNXSchema] = [
     _unary("Transpose", 1, "data", "transposed", types=_ANY, attributes=[ONNXAttribute("perm", _A.Ints)]),
     _unary("Flatten", 11, "input", "output", types=_ANY, attributes=[ONNXAttribute("axis", _A.Int, 1)]),
     _unary("Identity", 1, "input", "output", types=_ANY),
+    # Not an ONNX operator: the node the fusion pass puts in place of MatMul -> scale -> Softmax -> MatMul.
+    ONNXSchema("FusedAttention", 1,
+               [ONNXParameter("Q", "T"), ONNXParameter("K", "T"), ONNXParameter("V", "T")], [ONNXParameter("O", "T")],
+               [ONNXAttribute("scale", _A.Float, 1.0)], [ONNXTypeConstraint("T", [dace.float32])],
+               "softmax(scale * Q K^T) V per batch entry; Q, O are [..., Sq, D], K, V are [..., Sk, D]."),
     ONNXSchema("Pow", 12, [ONNXParameter("X", "T"), ONNXParameter("Y", "T1")], [ONNXParameter("Z", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64]), ONNXTypeConstraint("T1", _NUMERIC)]),
     ONNXSchema("ReduceMean", 11, [ONNXParameter("data", "T")], [ONNXParameter("reduced", "T")],

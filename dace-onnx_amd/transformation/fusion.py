@@ -24,6 +24,8 @@ MatMul -> Transpose -> Reshape               MatMul writes the final array throu
 ReduceMean, Sub, Pow(2), ReduceMean,         LayerNormalization (what exporters below
 Add(eps), Sqrt, Div, Mul(gamma), Add(beta)   opset 17 write for ``nn.LayerNorm``)
 Div(sqrt 2), Erf, Add(1), Mul(x), Mul(0.5)   Gelu (exact erf form, any operand order)
+MatMul(alpha) -> Softmax(last) -> MatMul     FusedAttention when the kernel supports the
+                                             shape (128 keys, head size 64)
 MatMuls of one A with constant weights       one MatMul with the weights (and biases)
 (the Q, K, V projections)                    concatenated along N; the readers
                                              address their slice of the wide result
@@ -600,6 +602,71 @@ def _fuse_decomposed_gelu(sdfg: SDFG, state: SDFGState) -> int:
     return fused
 
 
+# ----------------------------------------------------------------------------- attention
+def _fuse_attention(sdfg: SDFG, state: SDFGState) -> int:
+    """scores = alpha * (Q K^T); probs = Softmax(scores, last axis); ctx = probs V, every
+    intermediate single-use, becomes one FusedAttention node that reads Q, K, V and
+    writes ctx through the views the two MatMuls already carry. Runs after the view
+    folds (so K^T and the head split are strides) and before the projections are
+    widened (which only rebases those views)."""
+    from ..onnx.nodes.onnx_op import get_onnx_node
+    from ..onnx.op_implementations.mi355x_implementations import MI355XFusedAttention
+    fused = 0
+    for sm in list(state.nodes()):
+        if sm not in state.nodes() or not _is_op(sm, "Softmax"):
+            continue
+        s_in, probs = _in_edge(state, sm, "input"), _out_access(state, sm, "output")
+        if s_in is None or probs is None or not isinstance(s_in.src, AccessNode):
+            continue
+        scores = s_in.src
+        rank = len(sdfg.arrays[scores.data].shape)
+        if rank < 2 or sm.axis % rank != rank - 1 or _single_consumer(sdfg, state, scores) is None:
+            continue
+        prod1 = _producer(state, scores)
+        use2 = _next_op(sdfg, state, probs, "MatMul")
+        if prod1 is None or not _is_op(prod1.src, "MatMul") or use2 is None or use2.dst_conn != "A":
+            continue
+        mm1, mm2 = prod1.src, use2.dst
+        if any(_in_edge(state, n, c) is not None for n in (mm1, mm2) for c in ("_bias", "_residual")) \
+                or any(getattr(n, "_activation", None) for n in (mm1, mm2)) \
+                or getattr(mm1, "_y_view", None) or getattr(mm2, "_a_view", None) or getattr(mm2, "_alpha", 1.0) != 1.0:
+            continue
+        q_e, kt_e, v_e, o_e = _in_edge(state, mm1, "A"), _in_edge(state, mm1, "B"), _in_edge(state, mm2, "B"), \
+            _out_edge(state, mm2, "Y")
+        if None in (q_e, kt_e, v_e, o_e) or not all(isinstance(e.src, AccessNode) for e in (q_e, kt_e, v_e)):
+            continue
+
+        def view_of(edge, node, attr):
+            v = getattr(node, attr, None)
+            if v:
+                return [list(v[0]), list(v[1]), int(v[2]) if len(v) > 2 else 0]
+            d = sdfg.arrays[edge.data.data]
+            return [list(d.shape), list(d.strides), 0]
+
+        qv, ktv = view_of(q_e, mm1, "_a_view"), view_of(kt_e, mm1, "_b_view")
+        vv, ov = view_of(v_e, mm2, "_b_view"), view_of(o_e, mm2, "_y_view")
+        if len(ktv[0]) < 2:
+            continue
+        kv = [ktv[0][:-2] + [ktv[0][-1], ktv[0][-2]], ktv[1][:-2] + [ktv[1][-1], ktv[1][-2]], ktv[2]]  # K = (K^T)^T
+        f32 = sdfg.arrays[q_e.data.data].dtype
+        plan = MI355XFusedAttention._plan([(Array(f32, v[0], v[1]), v[2]) for v in (qv, kv, vv, ov)])
+        if plan is None or plan[3] != MI355XFusedAttention.SUPPORTED_KEYS or plan[4] != MI355XFusedAttention.SUPPORTED_HEAD:
+            continue
+        node = get_onnx_node("FusedAttention")(mm1.label + "_attention", scale=float(getattr(mm1, "_alpha", 1.0)))
+        state.add_node(node)
+        for conn, edge, view in (("Q", q_e, qv), ("K", kt_e, kv), ("V", v_e, vv)):
+            node.add_in_connector(conn)
+            state.add_edge(edge.src, None, node, conn, sdfg.make_array_memlet(edge.src.data))
+            setattr(node, "_" + conn.lower() + "_view", tuple(view))
+        node.add_out_connector("O")
+        node._o_view = tuple(ov)
+        out_access = o_e.dst
+        _drop_chain(sdfg, state, [mm1, sm, mm2], [q_e.src, kt_e.src, v_e.src, out_access])
+        state.add_edge(node, "O", out_access, None, sdfg.make_array_memlet(out_access.data))
+        fused += 1
+    return fused
+
+
 # ----------------------------------------------------------------------------- horizontal fusion
 def _rebase_strides(shape, strides, n_old, n_new):
     """A view (shape, strides) into a contiguous [rows, n_old] array, re-expressed
@@ -663,7 +730,8 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
         if any(isinstance(n, AccessNode) and n is not y_e.dst and n.data == y_e.dst.data for n in state.nodes()):
             continue
         readers = state.out_edges(y_e.dst)
-        if not readers or not all(_is_op(r.dst, "MatMul") and r.dst_conn in ("A", "B") for r in readers):
+        if not readers or not all((_is_op(r.dst, "MatMul") and r.dst_conn in ("A", "B")) or
+                                  (_is_op(r.dst, "FusedAttention") and r.dst_conn in ("Q", "K", "V")) for r in readers):
             continue
         if any(r.dst is node for r in readers):
             continue
@@ -695,7 +763,7 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
         for (node, a_e, b_e, bias_e, y_e, readers), width in zip(members, widths):
             ydesc = sdfg.arrays[y_e.dst.data]
             for r in readers:
-                attr = "_a_view" if r.dst_conn == "A" else "_b_view"
+                attr = {"A": "_a_view", "B": "_b_view", "Q": "_q_view", "K": "_k_view", "V": "_v_view"}[r.dst_conn]
                 old = getattr(r.dst, attr, None)
                 shape, strides = (old[0], old[1]) if old else (list(ydesc.shape), list(ydesc.strides))
                 offset = old[2] if old and len(old) > 2 else 0
@@ -711,6 +779,14 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
         for r, attr, view in rewires:
             trial.setdefault(r.dst, {})[attr] = view
         for consumer, views in trial.items():
+            if _is_op(consumer, "FusedAttention"):
+                from ..onnx.op_implementations.mi355x_implementations import MI355XFusedAttention
+                cur = [views.get(a, getattr(consumer, a)) for a in ("_q_view", "_k_view", "_v_view", "_o_view")]
+                plan = MI355XFusedAttention._plan([(Array(y0.dtype, v[0], v[1]), v[2]) for v in cur])
+                if plan is None or plan[3] != MI355XFusedAttention.SUPPORTED_KEYS or plan[4] != MI355XFusedAttention.SUPPORTED_HEAD:
+                    ok = False
+                continue
+
             def operand(conn, attr):
                 v = views.get(attr, getattr(consumer, attr, None))
                 if v:
@@ -794,6 +870,7 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
         total += _fold_into_contractions(sdfg, state)
         total += _fold_views(sdfg, state)
         _remove_dead_nodes(sdfg, state)  # folded Reshape/Transpose chains must not count as readers
+        total += _fuse_attention(sdfg, state)
         total += _fuse_shared_input_matmuls(sdfg, state)
         total += _pretranspose_weights(sdfg, state)
         _remove_dead_nodes(sdfg, state)

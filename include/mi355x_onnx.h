@@ -126,6 +126,23 @@ int mi355x_softmax_f32(const float* X, float* Y,
                        int64_t outer, int64_t axis_len, int64_t inner,
                        void* stream);
 
+/* Scaled-dot-product attention core, fp32, one launch:
+ *   O[b0,b1] = softmax(scale * Q[b0,b1] K[b0,b1]^T, over keys) V[b0,b1]
+ * Q, O are [Sq, D], K, V are [Sk, D] per (b0, b1) slice; the last dimension is
+ * contiguous, *_strides = {batch0, batch1, row} element strides (multiples of 4,
+ * operands 16-byte aligned), so the head split/merge of a [B, S, H*D] projection is
+ * expressed without a copy. Replaces the node sequence MatMul -> (Div | Mul by a
+ * scalar) -> Softmax(last axis) -> MatMul that the reference expands one node at a
+ * time (pure_implementations.py:130-235, 346-366); the score tensor never reaches
+ * memory. Supported: Sk == 128, D == 64; anything else returns
+ * MI355X_ERR_INVALID_ARGUMENT and launches nothing (the caller keeps the three
+ * separate nodes). */
+int mi355x_attention_f32(const float* Q, const float* K, const float* V, float* O,
+                         int64_t batch0, int64_t batch1, int64_t Sq, int64_t Sk, int64_t D,
+                         const int64_t* q_strides, const int64_t* k_strides,
+                         const int64_t* v_strides, const int64_t* o_strides,
+                         float scale, void* stream);
+
 /* ONNX LayerNormalization over the last axis, fp32, X is [rows, cols]:
  *   y = (x - mean) / sqrt(var + eps) * gamma + beta, biased variance.
  * The reference has no such node (opset 12); it runs the exporter's

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from dace_onnx_amd import sdfg as dace
+from dace_onnx_amd import _lib, sdfg as dace
 import dace_onnx_amd.onnx as donnx
 from dace_onnx_amd.util import utils
 from oracle import pure_ops as O
@@ -206,6 +206,28 @@ def test_layer_normalization(shape, axis):
     Y2 = np.zeros_like(X)
     donnx.ONNXLayerNormalization(X=X, Scale=g, Y=Y2, axis=axis)  # no bias, default epsilon
     assert rel_err(O.layer_normalization(X, g, None, axis=axis, epsilon=1e-5), Y2) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("batch, sq", [((2, 3), 128), ((1, 5), 100), ((4, ), 16), ((1, 1), 1)])
+def test_fused_attention_c_abi(batch, sq):
+    # softmax(scale * Q K^T) V through the C ABI, operands as strided slices of one packed projection
+    rng = np.random.default_rng(31)
+    b0, b1 = (1, ) * (2 - len(batch)) + tuple(batch)
+    packed = torch.from_numpy(rng.normal(size=(b0, max(sq, 128), b1, 3, 64)).astype(np.float32)).cuda()
+    q, k, v = packed[:, :sq, :, 0], packed[:, :128, :, 1], packed[:, :128, :, 2]      # [b0, S, b1, 64] views
+    out = torch.zeros(b0, sq, b1, 64, device="cuda")
+    lib = _lib.library()
+    strides = lambda t: _lib.i64_array([t.stride(0), t.stride(2), t.stride(1)])
+    scale = 0.125
+    _lib.check(lib.mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq, 128, 64,
+                                        strides(q), strides(k), strides(v), strides(out), scale, _lib.current_stream()),
+               "mi355x_attention_f32")
+    Q, K, V = (t.permute(0, 2, 1, 3).cpu().numpy().astype(np.float64) for t in (q, k, v))
+    expected = O.matmul(O.softmax(O.matmul(Q, np.swapaxes(K, -1, -2)) * scale, axis=-1), V)
+    assert rel_err(expected, out.permute(0, 2, 1, 3).cpu().numpy()) < FP32_REL_TOL
+    # unsupported shapes are rejected, nothing is launched
+    assert lib.mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq, 64, 64,
+                                    strides(q), strides(k), strides(v), strides(out), scale, _lib.current_stream()) == 1
 
 
 # ----------------------------------------------------------------------------- elementwise

@@ -51,6 +51,22 @@ def test_fused_bert_layer_is_nine_launches():
     assert out[15] == 9 and ffn1[15] == 5 and ffn2[15] == 9
 
 
+def test_bert_base_attention_core_is_one_launch():
+    # 128 keys, head size 64: MatMul -> Div -> Softmax -> MatMul becomes the fused attention kernel, which reads
+    # Q, K, V as column slices of the wide projection and writes the heads merged
+    w = pure_ops.bert_layer_weights(np.random.default_rng(0), hidden=768, ffn=3072)
+    calls = _launches(donnx.ONNXModel("bert_base", bert_encoder_layer_model(w, 2, 128, 12)))
+    assert sorted(f for f, _ in calls) == ["mi355x_attention_f32"] + ["mi355x_gemm_f32"] * 4 + ["mi355x_layernorm_f32"] * 2
+    a = [args for f, args in calls if f == "mi355x_attention_f32"][0]
+    assert [x.offset for x in a[:4]] == [0, 768, 1536, 0]
+    assert a[4:9] == [2, 12, 128, 128, 64]
+    assert a[9] == a[10] == a[11] == [128 * 2304, 64, 2304] and a[12] == [128 * 768, 64, 768]
+    assert a[13] == pytest.approx(0.125)
+    # 64 keys: not a shape the kernel supports, the three nodes stay
+    calls = _launches(donnx.ONNXModel("bert_s64", bert_encoder_layer_model(w, 2, 64, 12)))
+    assert [f for f, _ in calls].count("mi355x_attention_f32") == 0 and len(calls) == 9
+
+
 def test_shared_input_matmuls_with_other_readers_are_left_alone():
     # Y1 is also read by an Add: a column slice of a wide result cannot feed it without a copy
     rng = np.random.default_rng(1)
