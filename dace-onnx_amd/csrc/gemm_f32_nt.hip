@@ -68,9 +68,9 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     const int wm = wave % WAVES_M, ks = wave / WAVES_M;   // wave row, k-split group
 
     const int64_t logical = xcd_remap(blockIdx.x, p.nwg);
-    const int64_t tiles_per_batch = p.tiles_m * p.tiles_n;
-    const int64_t b = logical / tiles_per_batch, t = logical % tiles_per_batch;
-    const int64_t b0 = b / p.batch1, b1 = b % p.batch1;
+    const uint32_t tiles_per_batch = (uint32_t)(p.tiles_m * p.tiles_n);
+    const uint32_t b = (uint32_t)logical / tiles_per_batch, t = (uint32_t)logical % tiles_per_batch;
+    const int64_t b0 = b / (uint32_t)p.batch1, b1 = b % (uint32_t)p.batch1;
     int64_t tm, tn;
     tile_coords(t, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
     const int64_t m0 = tm * BM, n0 = tn * BN;
@@ -185,6 +185,23 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         load_a(ra[r], r);
         load_b(rb[r], r);
     }
+    // The small-tile variants have registers to spare: fetch this lane's bias and residual
+    // values now, so the epilogue does not wait for two more trips to memory (k-split
+    // group 1 never needs them).
+    constexpr bool PREFETCH_EPI = KSPLIT == 2 && TN <= 4;
+    f32x4 pre_bias[PREFETCH_EPI ? TN : 1], pre_res[PREFETCH_EPI ? TN : 1];
+    if constexpr (PREFETCH_EPI) {
+        const int64_t pm = m0 + 16 * wm + li;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int64_t n = n0 + 16 * j + 4 * lq;
+            const bool in = ks == 0 && pm < p.M && n < p.N;
+            pre_bias[j] = (in && (p.epi & MI355X_EPI_BIAS)) ? *reinterpret_cast<const f32x4*>(p.bias + n) : f32x4{0.f, 0.f, 0.f, 0.f};
+            pre_res[j] = (in && (p.epi & MI355X_EPI_RESIDUAL))
+                             ? *reinterpret_cast<const f32x4*>(p.residual + b0 * p.r_sb0 + b1 * p.r_sb1 + pm * p.r_sm + n)
+                             : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
     store_b(rb[0], 0);
     store_b(rb[1], 1);
     __syncthreads();
@@ -226,12 +243,14 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         if (n >= p.N) continue;
         f32x4 v = acc[j] * p.alpha;
         f32x4 bv = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (p.epi & MI355X_EPI_BIAS) bv = *reinterpret_cast<const f32x4*>(p.bias + n);
+        if constexpr (PREFETCH_EPI) bv = pre_bias[j];
+        else if (p.epi & MI355X_EPI_BIAS) bv = *reinterpret_cast<const f32x4*>(p.bias + n);
         v.x = apply_epilogue(v.x, p.epi, bv.x);
         v.y = apply_epilogue(v.y, p.epi, bv.y);
         v.z = apply_epilogue(v.z, p.epi, bv.z);
         v.w = apply_epilogue(v.w, p.epi, bv.w);
-        if (R) v += *reinterpret_cast<const f32x4*>(R + m * p.r_sm + n);
+        if constexpr (PREFETCH_EPI) v += pre_res[j];
+        else if (R) v += *reinterpret_cast<const f32x4*>(R + m * p.r_sm + n);
         *reinterpret_cast<f32x4*>(C + m * p.c_sm + n) = v;
     }
 }
@@ -240,15 +259,15 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
 // and N a multiple of 4. Additionally needed here: K a multiple of the 32-k tile.
 bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.K % NT_BK != 0 || p.K == 0) return false;
-    // Candidates: 64x48 and 64x64 tiles with two k-split groups, 128x96 tiles without.
+    // Candidates: 64x48, 64x64 and 64x144 tiles with two k-split groups, 128x96 tiles without.
     // Cost ~ rounds of workgroups over the CUs x tile area, the large tile discounted
     // for needing half the L2 traffic per FLOP and no reduction.
     struct Cand { int bm, bn; double weight; };
-    const Cand cands[] = {{64, 48, 1.0}, {64, 64, 1.0}, {128, 96, 0.8}};
+    const Cand cands[] = {{64, 48, 1.0}, {64, 64, 1.0}, {128, 96, 0.8}, {64, 144, 0.9}};
     int best = 0;
     double best_cost = 1e300;
     const char* force = getenv("MI355X_GEMM_NT_BN");
-    for (int c = 0; c < 3; ++c) {
+    for (int c = 0; c < 4; ++c) {
         const int64_t nwg = p.batch * ceil_div(p.M, cands[c].bm) * ceil_div(p.N, cands[c].bn);
         const double cost = (double)ceil_div(nwg, (int64_t)cus) * cands[c].bm * cands[c].bn * cands[c].weight;
         if (force ? atoi(force) == cands[c].bn : cost < best_cost) { best = c; best_cost = cost; if (force) break; }
@@ -264,7 +283,8 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
     if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
+    else if (best == 2) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_f32_nt_kernel<9, 4, 2>), grid, block, 0, stream, p);
     return true;
 }
 

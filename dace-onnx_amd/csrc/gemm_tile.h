@@ -12,22 +12,26 @@ constexpr int LDS_PAD = 4;
 
 // Hardware places workgroup w on XCD w % 8. Give XCD x the contiguous logical
 // range it would own if the tile space were cut into eight slabs.
+// (Grids are below 2^31 workgroups: 32-bit arithmetic, a 64-bit division costs
+// every wave several hundred instructions before its first load.)
 __device__ __forceinline__ int64_t xcd_remap(int64_t wg, int64_t nwg) {
-    const int64_t full = nwg / NUM_XCD, rem = nwg % NUM_XCD;
-    const int64_t xcd = wg % NUM_XCD, slot = wg / NUM_XCD;
-    return xcd * full + (xcd < rem ? xcd : rem) + slot;
+    const uint32_t w = (uint32_t)wg, n = (uint32_t)nwg;
+    const uint32_t full = n / NUM_XCD, rem = n % NUM_XCD;
+    const uint32_t xcd = w % NUM_XCD, slot = w / NUM_XCD;
+    return (int64_t)(xcd * full + (xcd < rem ? xcd : rem) + slot);
 }
 
 // Tile t of a tiles_m x tiles_n grid, walked in panels of group_m tile rows, down
 // the panel's rows first. Consecutive t (the slab one XCD works on at a time, see
 // xcd_remap) then cover a group_m x (slab / group_m) block of tiles instead of a
 // single tile row, so the XCD's L2 fetches far fewer distinct operand rows.
-__device__ __forceinline__ void tile_coords(int64_t t, int64_t tiles_m, int64_t tiles_n, int group_m,
+__device__ __forceinline__ void tile_coords(int64_t t64, int64_t tiles_m64, int64_t tiles_n64, int group_m,
                                             int64_t& tm, int64_t& tn) {
-    const int64_t panel = group_m * tiles_n;
-    const int64_t first_m = (t / panel) * group_m;
-    const int64_t rows = tiles_m - first_m < group_m ? tiles_m - first_m : group_m;
-    const int64_t in_panel = t % panel;
+    const uint32_t t = (uint32_t)t64, tiles_m = (uint32_t)tiles_m64, tiles_n = (uint32_t)tiles_n64;
+    const uint32_t panel = (uint32_t)group_m * tiles_n;
+    const uint32_t first_m = (t / panel) * (uint32_t)group_m;
+    const uint32_t rows = tiles_m - first_m < (uint32_t)group_m ? tiles_m - first_m : (uint32_t)group_m;
+    const uint32_t in_panel = t % panel;
     tm = first_m + in_panel % rows;
     tn = in_panel / rows;
 }
