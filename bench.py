@@ -32,6 +32,10 @@ if ROOT not in sys.path:
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_INT8_MFMA_TOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+# L2 <-> fabric bytes of the four GEMM launches of one layer, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script scaled by a copy kernel of known size (profiles/bert_layer_gemm_traffic.txt); counters cannot be
+# read from inside the process, so the figure is carried here and re-measured whenever the GEMM kernels change
+GEMM_TRAFFIC_BYTES_PER_LAYER = 193451535
 
 
 def graph_time_us(launch, reps=50, replays=5):
@@ -201,7 +205,7 @@ def main():
 
     # ---- per-kernel durations, HIP events on the launch stream -----------------------------
     kernels = []
-    gemm_flops = gemm_us = 0.0
+    gemm_flops = gemm_us = gemm_bytes = 0.0
     if not args.no_kernels:
         for node, relaunch in compiled.bound_launches():
             name = node.function
@@ -210,6 +214,7 @@ def main():
             us = graph_time_us(relaunch)
             if name == "mi355x_gemm_f32":
                 gemm_flops += flops
+                gemm_bytes += nbytes
                 gemm_us += us
                 label = "gemm_f32 b{}x{} {}x{}x{} epi={}".format(*plain[5:10], plain[15])
                 kernels.append(kernel_row(label, us, flops, nbytes, "mfma"))
@@ -257,7 +262,8 @@ def main():
     if gemm_us > 0:
         achieved = gemm_flops / gemm_us / 1e6
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                    "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES_PER_LAYER,
+                    "algorithmic_bytes_per_layer": gemm_bytes,
                     "kernel": "gemm_f32_nt_kernel (all mi355x_gemm_f32 launches of one layer: QKV, output projection, FFN1, "
                               "FFN2; the attention core runs in its own fused kernel, listed under kernels)",
                     "flop_per_layer": gemm_flops, "us_per_layer": round(gemm_us, 2)}
