@@ -1,0 +1,98 @@
+"""DaceModule: nn.Module -> ONNX graph -> "mi355x" expansions (the reference's tests/pytorch/
+test_bert_encoder.py, test_module_conv-style checks). Host-side structure without a GPU, results
+against the module itself evaluated in float64 on the CPU with one."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from dace_onnx_amd import sdfg as dace
+from dace_onnx_amd.pytorch import DaceModule, dace_module, module_to_onnx, UnsupportedModule
+from dace_onnx_amd.testing.utils import torch_tensors_close
+from conftest import rel_err, FP32_REL_TOL
+
+
+def _bert_layer(hidden=768, heads=12, ffn=3072):
+    from transformers import BertConfig
+    from transformers.models.bert.modeling_bert import BertLayer
+    cfg = BertConfig(hidden_size=hidden, num_attention_heads=heads, intermediate_size=ffn, hidden_act="gelu",
+                     layer_norm_eps=1e-12, attention_probs_dropout_prob=0.0, hidden_dropout_prob=0.0)
+    cfg._attn_implementation = "eager"
+    torch.manual_seed(0)
+    return BertLayer(cfg).eval()
+
+
+def _functions(dm):
+    return [n.function for n, _ in dm.dace_model.expand().all_nodes_recursive() if isinstance(n, dace.KernelCall)]
+
+
+def test_sequential_is_written_in_the_exporters_vocabulary():
+    m = nn.Sequential(nn.Linear(8, 16), nn.GELU(), nn.LayerNorm(16), nn.Dropout(0.1), nn.Linear(16, 4), nn.Softmax(dim=-1))
+    ops = [n.op_type for n in module_to_onnx(m, (torch.randn(5, 8), )).graph.node]
+    assert ops == ["Gemm", "Div", "Erf", "Add", "Mul", "Mul", "ReduceMean", "Sub", "Pow", "ReduceMean", "Add", "Sqrt",
+                   "Div", "Mul", "Add", "Gemm", "Softmax"]
+    names = {i.name for i in module_to_onnx(m, (torch.randn(5, 8), )).graph.initializer}
+    assert {"0.weight", "0.bias", "2.weight", "2.bias", "4.weight", "4.bias"} <= names   # parameter names survive
+    dm = DaceModule(m, dummy_inputs=(torch.randn(5, 8), ))
+    assert sorted(_functions(dm)) == ["mi355x_gemm_f32", "mi355x_gemm_f32", "mi355x_layernorm_f32", "mi355x_softmax_f32"]
+
+
+def test_transformers_bert_layer_becomes_seven_launches():
+    dm = DaceModule(_bert_layer(), dummy_inputs=(torch.randn(2, 128, 768), ))
+    fns = _functions(dm)
+    assert sorted(fns) == ["mi355x_attention_f32"] + ["mi355x_gemm_f32"] * 4 + ["mi355x_layernorm_f32"] * 2
+
+
+def test_unsupported_modules_and_modes_are_refused():
+    with pytest.raises(UnsupportedModule, match="LSTM"):
+        module_to_onnx(nn.LSTM(4, 4), (torch.randn(2, 3, 4), ))
+    with pytest.raises(UnsupportedModule, match="tanh"):
+        module_to_onnx(nn.GELU(approximate="tanh"), (torch.randn(2, 4), ))
+    with pytest.raises(UnsupportedModule, match="group"):
+        module_to_onnx(nn.Conv2d(4, 4, 3, groups=2), (torch.randn(1, 4, 8, 8), ))
+    with pytest.raises(NotImplementedError, match="inference only"):
+        DaceModule(nn.ReLU(), backward=True)
+
+
+@pytest.mark.gpu
+def test_bert_encoder_layer_module():
+    # the reference's test_bert_encoder.py: DaceModule(BertLayer) against the PyTorch module
+    layer = _bert_layer()
+    x = torch.randn(8, 128, 768)
+    with torch.no_grad():
+        ref = layer.double()(x.double())
+        ref = ref[0] if isinstance(ref, (tuple, list)) else ref
+    dace_layer = DaceModule(layer.float())
+    got = dace_layer(x.cuda())
+    assert got.is_cuda and got.dtype == torch.float32
+    assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL
+    torch_tensors_close("output", ref.float(), got.cpu(), rtol=1e-4, atol=1e-4)
+    assert dace_layer.dace_model.compile_and_init().num_launches == 7
+    with pytest.raises(TypeError, match="was built for"):
+        dace_layer(torch.randn(4, 128, 768).cuda())
+
+
+@pytest.mark.gpu
+def test_conv_relu_linear_module_and_decorator():
+    @dace_module
+    class Net(nn.Sequential):
+        def __init__(self):
+            super().__init__(nn.Conv2d(32, 48, 3, padding=1), nn.ReLU(), nn.Conv2d(48, 16, 1, stride=2, bias=False),
+                             nn.Flatten(), nn.Linear(16 * 6 * 6, 40), nn.ReLU(), nn.Linear(40, 10), nn.Softmax(dim=1))
+
+    torch.manual_seed(1)
+    net = Net()
+    assert isinstance(net, DaceModule)
+    x = torch.randn(6, 32, 12, 12)
+    with torch.no_grad():
+        ref = copy.deepcopy(net.model).double()(x.double())
+    got = net(x.cuda())
+    assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL
+    # parameters changed after the graph was built: rebuilt on request
+    with torch.no_grad():
+        net.model[6].bias.add_(1.0)
+        ref2 = copy.deepcopy(net.model).double()(x.double())
+    net.reset_sdfg()
+    assert rel_err(ref2.numpy(), net(x.cuda()).cpu().numpy()) < FP32_REL_TOL
