@@ -295,3 +295,26 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(base, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), os.path.join(base, f)
+
+
+def test_daceml_adapter_mirrors_nodes_and_needs_the_real_packages():
+    from dace_onnx_amd import daceml_adapter
+    # the mirror runs on anything with the SDFG attribute surface; on this package's own objects it must
+    # reproduce the direct expansion (same C++ tasklet text)
+    node = donnx.ONNXMatMul("Matmul")
+    sdfg, st = _one_node_sdfg(node, {"A": ([8, 128, 768], dace.float32), "B": ([768, 3072], dace.float32)},
+                              {"Y": ([8, 128, 3072], dace.float32)})
+    call = daceml_adapter.mirror_expansion(node, st, sdfg)
+    assert call.function == "mi355x_gemm_f32"
+    assert "mi355x_gemm_f32(_A, _B, _Y, nullptr, nullptr, 1, 1, 1024, 3072, 768" in call.as_cpp()
+    conv = donnx.ONNXConv("Conv", strides=[2, 2])
+    sdfg, st = _one_node_sdfg(conv, {"X": ([5, 3, 10, 10], dace.float32), "W": ([16, 3, 3, 3], dace.float32)},
+                              {"Y": ([5, 16, 4, 4], dace.float32)})
+    cpp = daceml_adapter.mirror_expansion(conv, st, sdfg).as_cpp()
+    assert "mi355x_conv2d_f32(_X, _W, nullptr, _Y, 5, 3, 10, 10, 16, 3, 3" in cpp and "__dace_current_stream" in cpp
+    # a node the implementation refuses (1-D operand) mirrors to None: the adapter then falls back like the reference
+    mm = donnx.ONNXMatMul("Matmul1d")
+    sdfg, st = _one_node_sdfg(mm, {"A": ([4], dace.float32), "B": ([4, 3], dace.float32)}, {"Y": ([3], dace.float32)})
+    assert daceml_adapter.mirror_expansion(mm, st, sdfg) is None
+    with pytest.raises(ImportError, match="dace"):
+        daceml_adapter.register()
