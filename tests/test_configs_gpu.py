@@ -256,3 +256,37 @@ def test_strided_gemm_head_split_merge_without_copies():
     vh = v.view(B_, S, Hh, D).permute(0, 2, 1, 3).double()
     ref = (probs.double() @ vh).permute(0, 2, 1, 3).reshape(B_, S, Hh * D)
     assert rel_err(ref.cpu().numpy(), ctx.cpu().numpy()) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- GEMM kernel variants, ragged shapes
+@pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144"])
+@pytest.mark.parametrize("M, N, K, epi", [(64, 48, 32, 0), (1, 4, 32, 1), (130, 52, 64, 9), (257, 100, 96, 5), (200, 148, 160, 3),
+                                          (1024, 768, 768, 9), (63, 764, 224, 8)])
+def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
+    """Both operands k-contiguous (activations x [N, K] weights): every tile variant of that kernel on shapes that
+    leave partial tiles in M and N, with each epilogue combination (1 bias, 2 relu, 4 gelu, 8 residual) and alpha."""
+    if tile == "auto":
+        monkeypatch.delenv("MI355X_GEMM_NT_BN", raising=False)
+    else:
+        monkeypatch.setenv("MI355X_GEMM_NT_BN", tile)
+    lib = _lib.library()
+    rng = np.random.default_rng(M * 7 + N * 3 + K + epi)
+    a = torch.from_numpy(rng.normal(size=(2, M, K)).astype(np.float32)).cuda()
+    w = torch.from_numpy(rng.normal(size=(N, K)).astype(np.float32)).cuda()          # [N, K]: B[k, n] = w[n, k]
+    bias = torch.from_numpy(rng.normal(size=N).astype(np.float32)).cuda()
+    res = torch.from_numpy(rng.normal(size=(2, M, N)).astype(np.float32)).cuda()
+    out = torch.full((2, M, N), float("nan"), device="cuda")
+    alpha = 0.5
+    _lib.check(lib.mi355x_gemm_f32(a.data_ptr(), w.data_ptr(), out.data_ptr(), bias.data_ptr(), res.data_ptr(), 1, 2, M, N, K,
+                                   _lib.i64_array([0, M * K, K, 1]), _lib.i64_array([0, 0, 1, K]), _lib.i64_array([0, M * N, N]),
+                                   _lib.i64_array([0, M * N, N]), alpha, epi, _lib.current_stream()), "gemm")
+    ref = alpha * (a.double() @ w.double().T)
+    if epi & 1:
+        ref = ref + bias.double()
+    if epi & 2:
+        ref = torch.relu(ref)
+    if epi & 4:
+        ref = torch.nn.functional.gelu(ref)
+    if epi & 8:
+        ref = ref + res.double()
+    assert rel_err(ref.cpu().numpy(), out.cpu().numpy()) < FP32_REL_TOL
