@@ -261,7 +261,7 @@ def test_strided_gemm_head_split_merge_without_copies():
 # ----------------------------------------------------------------------------- GEMM kernel variants, ragged shapes
 @pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144"])
 @pytest.mark.parametrize("M, N, K, epi", [(64, 48, 32, 0), (1, 4, 32, 1), (130, 52, 64, 9), (257, 100, 96, 5), (200, 148, 160, 3),
-                                          (1024, 768, 768, 9), (63, 764, 224, 8)])
+                                          (1024, 768, 768, 9), (63, 764, 224, 8), (100, 52, 2112, 9)])   # last: 64-k tiles
 def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
     """Both operands k-contiguous (activations x [N, K] weights): every tile variant of that kernel on shapes that
     leave partial tiles in M and N, with each epilogue combination (1 bias, 2 relu, 4 gelu, 8 residual) and alpha."""
