@@ -140,7 +140,7 @@ def main():
     lib = _lib.library()
     torch.cuda.set_device(0)
 
-    # ---- workload: BASELINE config 3 -------------------------------------------------
+    # ---- workload: benchmark config 3 -------------------------------------------------
     B, S, H, HEADS, FFN = 8, 128, 768, 12, 3072
     rng = np.random.default_rng(3)
     weights = pure_ops.bert_layer_weights(rng, hidden=H, ffn=FFN)
@@ -228,7 +228,7 @@ def main():
                                                                                      else plain[4:6]))
                 kernels.append(kernel_row(label, us, 0.0, nbytes, "hbm"))
 
-        # stand-alone configurations of the metric (BASELINE configs 2, 4, 5)
+        # stand-alone configurations of the metric (benchmark configs 2, 4, 5)
         st = _lib.current_stream
         xs = torch.randn(12288, 128, device="cuda")
         ys = torch.empty_like(xs)
@@ -287,7 +287,7 @@ def main():
         "value": round(ms_per_step, 5), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "BASELINE config 3: BERT-base encoder layer, B=8 S=128 H=768 heads=12 FFN=3072, "
+        "config": {"workload": "BASELINE.json configs[2]: BERT-base encoder layer, B=8 S=128 H=768 heads=12 FFN=3072, "
                                "ONNX graph of MatMul/Add/Reshape/Transpose/Div/Softmax/LayerNormalization/Gelu",
                    "launches_per_step": compiled.num_launches, "replay": "host_launches" if mode == "eager" else "hip_graph",
                    "max_rel_err_vs_oracle": err},

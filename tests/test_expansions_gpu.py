@@ -104,7 +104,7 @@ def test_conv_simple(num_in_channels, kernel_size, num_filters, bias):
 
 
 def test_conv_config1_stride2():
-    # BASELINE config 1 and the reference's README example (examples/plot_conv.py:43-46)
+    # benchmark config 1 (5x3x10x10 input, 16 filters 3x3, stride 2) and the reference's README example (examples/plot_conv.py:43-46)
     rng = np.random.default_rng(1)
     X = rng.random((5, 3, 10, 10), dtype=np.float32)
     W = rng.random((16, 3, 3, 3), dtype=np.float32)
