@@ -240,6 +240,18 @@ def main():
         us = graph_time_us(lambda: lib.mi355x_layernorm_f32(xl.data_ptr(), g_.data_ptr(), b_.data_ptr(), yl.data_ptr(),
                                                             1024, 768, 1e-12, st()))
         kernels.append(kernel_row("cfg2 layernorm 8x128x768", us, 0.0, 6297600.0, "hbm"))
+        # the same two kernels on inputs large enough that the 1.75 us launch floor no longer matters (805 MB each)
+        xs = torch.randn(1572864, 128, device="cuda")
+        ys = torch.empty_like(xs)
+        us = graph_time_us(lambda: lib.mi355x_softmax_f32(xs.data_ptr(), ys.data_ptr(), 1572864, 128, 1, st()), reps=5)
+        kernels.append(kernel_row("softmax 1572864x128 (1.6 GB moved)", us, 0.0, 8.0 * 1572864 * 128, "hbm"))
+        del xs, ys
+        xl = torch.randn(131072, 768, device="cuda")
+        yl = torch.empty_like(xl)
+        us = graph_time_us(lambda: lib.mi355x_layernorm_f32(xl.data_ptr(), g_.data_ptr(), b_.data_ptr(), yl.data_ptr(),
+                                                            131072, 768, 1e-12, st()), reps=5)
+        kernels.append(kernel_row("layernorm 131072x768 (0.8 GB moved)", us, 0.0, 8.0 * 131072 * 768, "hbm"))
+        del xl, yl
         xc = torch.randn(32, 64, 56, 56, device="cuda")
         wc = torch.randn(64, 64, 3, 3, device="cuda") * (2.0 / 576) ** 0.5
         bc = torch.zeros(64, device="cuda")
