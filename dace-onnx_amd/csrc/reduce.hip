@@ -42,9 +42,14 @@ __global__ __launch_bounds__(256) void reduce_mean_strided(const float* __restri
     if (idx >= outer * inner) return;
     const int64_t o = idx / inner, i = idx % inner;
     const float* x = X + o * axis_len * inner + i;
-    float s = 0.0f;
-    for (int64_t a = 0; a < axis_len; ++a) s += x[a * inner];
-    Y[idx] = s * inv_n;
+    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // independent chains, pairwise combination
+    int64_t a = 0;
+    for (; a + 8 <= axis_len; a += 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s[u] += x[(a + u) * inner];
+    }
+    for (int u = 0; a < axis_len; ++a, ++u) s[u] += x[a * inner];
+    Y[idx] = ((((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7])))) * inv_n;
 }
 
 }  // namespace mi355x
