@@ -440,223 +440,6 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
     }
 }
 
-// ---------------------------------------------------------------------------------------------
-// Persistent form of the gather kernel, for K / 32 a multiple of the look-ahead depth (K a multiple
-// of 192: every 3 x 3 convolution over a multiple of 64 channels, ...).
-//
-// With K of a few hundred a tile is only ~18 steps long and a workgroup that starts cold pays for a
-// launch, the decomposition of its positions, a look-ahead ring to fill and one trip to memory before
-// its first MFMA: measured, a third of the tile's time. Here the grid is one workgroup per slot of the
-// machine and a workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... as one stream of steps:
-// loads always run exactly one group of RING steps ahead, so during the last group of a tile they
-// already fetch the first group of the next tile, and the tile's results leave through
-// fire-and-forget stores while the next tile is multiplied. The step loop inside a tile is the same
-// branch-free loop as in the one-tile kernel; everything that happens once per tile (decoding the
-// next tile's positions, the k-split reduction, the epilogue) sits between two groups, once in the code.
-template <int TN>
-__global__ __launch_bounds__(CG_THREADS) void conv2d_f32_stream_kernel(ConvArgs p) {
-    constexpr int BM = CG_BM, BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
-    static_assert(BN % WAVE == 0, "a wave's loader units share their k-quad");
-    constexpr int UNITS = BN * (BK / 4);
-    static_assert(UNITS % CG_THREADS == 0, "whole units per thread");
-    constexpr int B_PER_T = UNITS / CG_THREADS;
-    constexpr int STAGE = BN * PITCH;
-    __shared__ __attribute__((aligned(16))) float lds[CG_STAGES * STAGE];
-    __shared__ __attribute__((aligned(16))) f32x4 lds_red[4 * TN * WAVE];   // partial sums of k-split group 1
-    __shared__ __attribute__((aligned(16))) uint32_t lds_tap[CG_MAX_K];     // see conv2d_f32_gather_kernel
-
-    const int tid = threadIdx.x;
-    const int lane = tid % WAVE, wave = tid / WAVE;
-    const int li = lane % 16, lq = lane / 16;
-    const int wm = wave % 4, ks = wave / 4;   // wave row, k-split group
-
-    for (int k = tid; k < p.K; k += CG_THREADS) {
-        const uint32_t c = fdiv((uint32_t)k, p.div_khw);
-        const uint32_t rs = (uint32_t)k - c * (uint32_t)(p.KH * p.KW);
-        const uint32_t r = fdiv(rs, p.div_kw);
-        const uint32_t t = rs - r * (uint32_t)p.KW;
-        lds_tap[k] = (rs << 27) | (c * (uint32_t)(p.H * p.Wd) + r * (uint32_t)(p.dil_h * p.Wd) + t * (uint32_t)p.dil_w);
-    }
-
-    const int groups = p.K / (BK * RING);   // K % (32 * RING) == 0 is a launch precondition
-    // tiles of this workgroup: blockIdx.x + i * gridDim.x (gridDim.x is a multiple of 8 or the tile count)
-    const int my_tiles = (int)((p.nwg - blockIdx.x + gridDim.x - 1) / gridDim.x);
-
-    // what the loaders need to know about a tile: the lane's W row, and this thread's output position
-    // (byte offset of its top-left input pixel, one bit per filter tap that falls into the pad)
-    struct TileState { const float* a_ptr; uint32_t xbase, tap_outside; int64_t m0, p0; };
-    const int p_local = tid % BN;
-    auto tile_state = [&](int i) __attribute__((always_inline)) {
-        TileState t;
-        const int64_t logical = xcd_remap((int64_t)blockIdx.x + (int64_t)i * gridDim.x, p.nwg);
-        int64_t tm, tn;
-        tile_coords(logical, p.tiles_m, p.tiles_p, p.group_m, tm, tn);
-        t.m0 = tm * BM;
-        t.p0 = tn * BN;
-        int64_t am = t.m0 + 16 * wm + li;
-        am = am < p.M ? am : p.M - 1;
-        t.a_ptr = p.W + am * p.K + 16 * ks + 4 * lq;
-        t.xbase = 0;
-        t.tap_outside = 0xffffffffu;
-        const int64_t pp = t.p0 + p_local;
-        if (pp < p.P) {
-            const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
-            const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
-            const uint32_t oy = fdiv(q, p.div_ow);
-            const uint32_t ox = q - oy * (uint32_t)p.OW;
-            const int iy0 = (int)oy * p.stride_h - p.pad_t;
-            const int ix0 = (int)ox * p.stride_w - p.pad_l;
-            t.xbase = (uint32_t)(((int)n * p.C * p.H * p.Wd + iy0 * p.Wd + ix0) * 4);
-            uint32_t outside = 0;
-            for (int r = 0; r < p.KH; ++r)
-                for (int c = 0; c < p.KW; ++c) {
-                    const bool ok = (unsigned)(iy0 + r * p.dil_h) < (unsigned)p.H && (unsigned)(ix0 + c * p.dil_w) < (unsigned)p.Wd;
-                    outside |= (ok ? 0u : 1u) << (r * p.KW + c);
-                }
-            t.tap_outside = outside;
-        }
-        return t;
-    };
-
-    int kq[B_PER_T], b_lds[B_PER_T];
-#pragma unroll
-    for (int it = 0; it < B_PER_T; ++it) {
-        kq[it] = __builtin_amdgcn_readfirstlane((tid + it * CG_THREADS) / BN);
-        b_lds[it] = p_local * PITCH + 4 * kq[it];
-    }
-
-    f32x4 acc[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    f32x4 ra[RING];            // W operand of step s in slot s % RING
-    f32x4 rb[RING][B_PER_T];   // gathered pixels of step s in slot s % RING
-    f32x4 bf[2][TN];           // X operands of step s in set s % 2
-
-    auto load_a = [&](f32x4& dst, const TileState& t, int kt) __attribute__((always_inline)) {
-        dst = *reinterpret_cast<const f32x4*>(t.a_ptr + (int64_t)kt * BK);
-    };
-    auto load_b = [&](f32x4 (&dst)[B_PER_T], const TileState& t, int kt) __attribute__((always_inline)) {
-        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.X), 0, p.x_bytes, 0x00020000);
-#pragma unroll
-        for (int it = 0; it < B_PER_T; ++it) {
-            const u32x4 taps = *reinterpret_cast<const u32x4*>(lds_tap + kt * BK + 4 * kq[it]);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const uint32_t off = t.xbase + ((taps[e] & 0x07ffffffu) << 2);
-                const uint32_t outside = (t.tap_outside >> (taps[e] >> 27)) & 1u;
-                dst[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(off | (outside << 31)), 0, 0));
-            }
-        }
-    };
-    auto store_b = [&](const f32x4 (&src)[B_PER_T], int stage) __attribute__((always_inline)) {
-#pragma unroll
-        for (int it = 0; it < B_PER_T; ++it) *reinterpret_cast<f32x4*>(lds + stage * STAGE + b_lds[it]) = src[it];
-    };
-    auto read_b = [&](f32x4 (&dst)[TN], int stage) __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-            dst[j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
-    };
-
-    // One group of RING steps. Step r multiplies slot r, loads the same position of the NEXT group
-    // (tile `nt`, k-tiles kt_next + r; for A the slot consumed one step earlier), writes the B tile two
-    // steps ahead to LDS and reads the operands one step ahead.
-    auto group = [&](const TileState& nt, int kt_next) __attribute__((always_inline)) {
-        cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) {
-            constexpr int r = decltype(r_tag)::value;
-            constexpr int cur = r & 1;  // RING is even: step parity == slot parity
-            load_b(rb[r], nt, kt_next + r);                      // slot r went to LDS two steps ago
-            // slot r - 1 was consumed in the previous step; at r == 0 that is slot RING - 1 of the group before,
-            // whose next-group load belongs to this group's target as well (kt_next + RING - 1 - RING + RING)
-            if constexpr (r > 0) load_a(ra[r - 1], nt, kt_next + r - 1);
-            store_b(rb[(r + 2) % RING], (r + 2) % CG_STAGES);    // two steps ahead
-            read_b(bf[cur ^ 1], (r + 1) % CG_STAGES);            // one step ahead, visible since the last barrier
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[cur][j][q], ra[r][q], acc[j], 0, 0, 0);
-            if constexpr (r == RING - 1) load_a(ra[r], nt, kt_next + r);   // the last slot, right after its use
-            constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
-            __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
-            __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(DS_RD, 1, 0);
-            }
-#pragma unroll
-            for (int v = 0; v < 4 * B_PER_T + 1; ++v) {
-                __builtin_amdgcn_sched_group_barrier(MFMA, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(VMEM_RD, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(MFMA, 4 * TN, 0);
-            __syncthreads();
-        });
-    };
-    static_assert(RING % 2 == 0 && RING % CG_STAGES == 0, "slot index fixes operand set and LDS buffer");
-
-    TileState cur_tile = tile_state(0);
-    __syncthreads();  // tap table complete
-#pragma unroll
-    for (int r = 0; r < RING; ++r) {
-        load_a(ra[r], cur_tile, r);
-        load_b(rb[r], cur_tile, r);
-    }
-    store_b(rb[0], 0);
-    store_b(rb[1], 1);
-    __syncthreads();
-    read_b(bf[0], 0);
-
-    for (int i = 0; i < my_tiles; ++i) {
-        // groups 0 .. groups - 2 of this tile: loads stay inside the tile
-        for (int g = 0; g + 1 < groups; ++g) group(cur_tile, (g + 1) * RING);
-        // last group: loads fetch the first group of the next tile (after the last tile: of the same tile
-        // again, cached data that nobody uses)
-        const TileState next_tile = i + 1 < my_tiles ? tile_state(i + 1) : cur_tile;
-        group(next_tile, 0);
-
-        // k-split group 1 hands its partial sums to group 0, which applies the epilogue and stores
-        if (ks == 1) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j) lds_red[(wm * TN + j) * WAVE + lane] = acc[j];
-        }
-        __syncthreads();   // the next write to lds_red is a whole tile of step barriers away
-        if (ks == 0) {
-            // acc[j][r] = Y[oc = m0 + 16 wm + li][p = p0 + 16 j + 4 lq + r]
-            const int64_t oc = cur_tile.m0 + 16 * wm + li;
-            const float bv = (oc < p.M && (p.epi & MI355X_EPI_BIAS)) ? p.bias[oc] : 0.f;
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int64_t pp = cur_tile.p0 + 16 * j + 4 * lq;
-                if (oc >= p.M || pp >= p.P) continue;
-                f32x4 v = acc[j] + lds_red[(wm * TN + j) * WAVE + lane];
-                v.x = apply_epilogue(v.x, p.epi, bv);
-                v.y = apply_epilogue(v.y, p.epi, bv);
-                v.z = apply_epilogue(v.z, p.epi, bv);
-                v.w = apply_epilogue(v.w, p.epi, bv);
-                if (p.vec_y) {
-                    const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
-                    const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
-                    __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(p.Y + ((int64_t)n * p.M + oc) * p.OHW + q));
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        if (pp + r >= p.P) break;
-                        const uint32_t n = fdiv((uint32_t)(pp + r), p.div_ohw);
-                        const uint32_t q = (uint32_t)(pp + r) - n * (uint32_t)p.OHW;
-                        p.Y[((int64_t)n * p.M + oc) * p.OHW + q] = v[r];
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        cur_tile = next_tile;
-    }
-}
-
 template <int BM, int BN, int BK, int WMs, int WNs>
 static void launch_conv(const ConvArgs& p, hipStream_t st) {
     const dim3 grid((unsigned)p.nwg), block(64 * WMs * WNs);
@@ -750,15 +533,6 @@ extern "C" int mi355x_conv2d_f32(const float* X, const float* W, const float* bi
         p.tiles_p = ceil_div(P, (int64_t)bn);
         p.nwg = p.tiles_m * p.tiles_p;
         MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "conv2d: grid too large");
-        if (K % (CG_BK * CG_RING) == 0 && !wide && !getenv("MI355X_CONV_NO_STREAM")) {
-            // persistent grid: every slot of the machine (a multiple of the XCD count), or one workgroup per tile
-            int64_t grid = (int64_t)2 * (cus / NUM_XCD) * NUM_XCD;
-            if (grid > p.nwg) grid = p.nwg;
-            const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = ceil_div(grid, (int64_t)NUM_XCD);
-            p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, CG_BM, bn);
-            hipLaunchKernelGGL(conv2d_f32_stream_kernel<4>, dim3((unsigned)grid), dim3(CG_THREADS), 0, st, p);
-            return check_launch("conv2d_f32_stream_kernel");
-        }
         if (wide) hipLaunchKernelGGL(conv2d_f32_gather_kernel<8>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
         else hipLaunchKernelGGL(conv2d_f32_gather_kernel<4>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
         return check_launch("conv2d_f32_gather_kernel");
