@@ -244,6 +244,22 @@ def test_binary_broadcast(op, a_shape, b_shape):
     assert np.array_equal(expected, C) or rel_err(expected, C) < 1e-6
 
 
+def test_gelu_dense_grid_absolute_error():
+    """The kernel's own erf (a fit, not the library routine) against the double-precision closed form on a
+    dense grid: the absolute error of Gelu stays within two fp32 roundings of the result."""
+    import math
+    X = np.linspace(-8.0, 8.0, 400001).astype(np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXGelu(X=X, Y=Y)
+    x64 = X.astype(np.float64)
+    ref = 0.5 * x64 * (1.0 + np.vectorize(math.erf)(x64 / math.sqrt(2.0)))
+    err = np.abs(Y.astype(np.float64) - ref)
+    assert err.max() <= 2 * np.spacing(np.float32(8.0)), err.max()
+    assert (err[np.abs(X) <= 1.0]).max() <= 2.5e-7
+    assert np.abs(Y[X <= -6.0]).max() <= 1e-6      # left tail goes to zero, not to garbage
+    assert Y[X == 0.0][0] == 0.0
+
+
 @pytest.mark.parametrize("shape", [(8, 16, 3072), (7, ), (1, 3, 5), (4097, )])
 def test_unary_ops(shape):
     X = np.random.default_rng(10).normal(scale=2, size=shape).astype(np.float32)
