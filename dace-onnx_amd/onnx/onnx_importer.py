@@ -73,6 +73,8 @@ class ONNXModel:
         :param infer_shapes: infer shapes of intermediate values; if ``False`` the model must carry
                              value_info for all of them.
         :param cuda: kept for signature compatibility; execution is always on the GPU.
+        :param fold_constants: replace nodes whose inputs are all constants by their value
+                               (``transformation/constant_folding.py``) before the graph is built.
         :param auto_optimize: apply the graph-level fusion pass before expanding (first call).
         :param parent_pytorch_module: when not None, weights whose names match parameters of this
                                       module are taken from it rather than from the ONNX graph.
@@ -88,6 +90,10 @@ class ONNXModel:
         self.do_auto_optimize = auto_optimize
         self.fuse = fuse
         self.use_hip_graph = use_hip_graph
+        model = self._constants_to_initializers(model)
+        if fold_constants:
+            from ..transformation.constant_folding import fold_constants as _fold
+            model = _fold(model)
         for node in model.graph.node:
             if not has_onnx_node(node.op_type):
                 raise ValueError("Unsupported ONNX operator: '{}'".format(node.op_type))
@@ -178,6 +184,49 @@ class ONNXModel:
         self._static_io = None
 
     # -- construction helpers ----------------------------------------------------------
+    @staticmethod
+    def _constants_to_initializers(model: ModelProto) -> ModelProto:
+        """``Constant`` nodes become weights at import, as in the reference
+        (``onnx_importer.py:193-229``, same checks and messages); here by turning each into an
+        initializer named after its output before anything else looks at the graph. The
+        caller's model is not modified."""
+        if not any(n.op_type == "Constant" for n in model.graph.node):
+            return model
+        import copy
+        model = copy.copy(model)
+        model.graph = copy.copy(model.graph)
+        possible_values = {"sparse_value", "value", "value_float", "value_floats", "value_int", "value_ints",
+                           "value_string", "value_strings"}
+        kept, extra = [], []
+        for node in model.graph.node:
+            if node.op_type != "Constant":
+                kept.append(node)
+                continue
+            attrs = {a.name: a for a in node.attribute}
+            if set(attrs).difference(possible_values):
+                raise ValueError(f"Got unexpected attributes on Constant node {set(attrs).difference(possible_values)}")
+            if len(attrs) != 1:
+                raise ValueError("Expected Constant node to have exactly one of its attributes set")
+            if len(node.input) != 0 or len(node.output) != 1:
+                raise ValueError("Expected Constant node to have no inputs and exactly 1 output")
+            (kind, attr), = attrs.items()
+            if kind == "value":
+                value = np.asarray(attr.value.array).reshape(attr.value.dims)
+            elif kind == "value_float":
+                value = np.asarray(attr.value, dtype=np.float32)
+            elif kind == "value_floats":
+                value = np.asarray(list(attr.value), dtype=np.float32)
+            elif kind == "value_int":
+                value = np.asarray(attr.value, dtype=np.int64)
+            elif kind == "value_ints":
+                value = np.asarray(list(attr.value), dtype=np.int64)
+            else:
+                raise ValueError(f"Constant node attribute '{kind}' is not supported")
+            extra.append(proto.numpy_helper.from_array(value, name=node.output[0]))
+        model.graph.node = kept
+        model.graph.initializer = list(model.graph.initializer) + extra
+        return model
+
     @staticmethod
     def _convert_attribute(attr):
         v = attr.value

@@ -6,20 +6,32 @@ ONNX graph on its first call (shapes taken from the actual inputs, or from
 module: ``parent_pytorch_module``, module.py:260-265), and from then on calls the
 compiled graph on device tensors.
 
-The reference obtains the ONNX graph from ``torch.onnx.export(opset_version=12)``
-(module.py:238-256). That exporter needs the ``onnx`` package, which is not a
-dependency here, so the graph is written directly from the module structure, in
-the same opset-12 vocabulary the exporter uses -- ``nn.Linear`` becomes Gemm
-(2-D input) or MatMul + Add, ``nn.LayerNorm`` the nine-node ReduceMean ... Add
-chain, ``nn.GELU`` the five-node Erf chain -- for the module types on the hot
-path: ``Sequential`` of Linear, Conv2d, ReLU, GELU, LayerNorm, Softmax, Flatten,
-Identity, Dropout (inference: identity), and ``transformers``' ``BertLayer``
-(the module of tests/pytorch/test_bert_encoder.py:17). Anything else raises
-``UnsupportedModule``. Inference only: ``backward=True`` is refused (the
-reference's autodiff is a separate subsystem).
+The reference obtains the ONNX graph from ``torch.onnx.export(opset_version=12,
+do_constant_folding=False, keep_initializers_as_inputs=True)`` (module.py:238-256).
+Two ways to the graph here (``exporter=``):
+
+* ``"structural"``: the graph is written directly from the module structure, in the
+  same opset-12 vocabulary the exporter uses -- ``nn.Linear`` becomes Gemm (2-D input)
+  or MatMul + Add, ``nn.LayerNorm`` the nine-node ReduceMean ... Add chain, ``nn.GELU``
+  the five-node Erf chain -- for the module types on the hot path: ``Sequential`` of
+  Linear, Conv2d, ReLU, GELU, LayerNorm, Softmax, Flatten, Identity, Dropout
+  (inference: identity), and ``transformers``' ``BertLayer`` (the module of
+  tests/pytorch/test_bert_encoder.py:17). Anything else raises ``UnsupportedModule``.
+* ``"torch"``: the reference's own call of the TorchScript exporter, any number of
+  inputs, any module whose exported operators have an ``ONNX<Op>`` node here. The
+  exporter's last step attaches onnxscript functions through the ``onnx`` package;
+  when that package is absent the step is skipped for the duration of the call (the
+  graphs concerned hold none).
+* ``"auto"`` (default): structural where it applies, the exporter otherwise.
+
+Inference only: ``backward=True`` is refused (the reference's autodiff is a separate
+subsystem).
 """
+import contextlib
+import io
 import math
 import typing
+import warnings
 from functools import wraps
 
 import numpy as np
@@ -188,6 +200,40 @@ def module_to_onnx(module: nn.Module, dummy_inputs: typing.Sequence[torch.Tensor
     return helper.make_model(graph, opset_imports=[helper.make_opsetid("", 12)])
 
 
+@contextlib.contextmanager
+def _exporter_without_onnx_package():
+    """The TorchScript exporter serializes the graph itself; only its final ``_add_onnxscript_fn`` step
+    imports ``onnx``. Without that package, replace the step by the identity while exporting."""
+    try:
+        import onnx  # noqa: F401
+        yield
+        return
+    except ImportError:
+        pass
+    from torch.onnx._internal.torchscript_exporter import onnx_proto_utils
+    saved = onnx_proto_utils._add_onnxscript_fn
+    onnx_proto_utils._add_onnxscript_fn = lambda model_bytes, custom_opsets: model_bytes
+    try:
+        yield
+    finally:
+        onnx_proto_utils._add_onnxscript_fn = saved
+
+
+def export_with_torch(module: nn.Module, dummy_inputs: typing.Sequence[torch.Tensor]) -> bytes:
+    """``torch.onnx.export`` with the reference's arguments (daceml/pytorch/module.py:238-256): opset 12, no
+    constant folding (folded weights lose the names that tie them to the module's parameters), initializers
+    kept as inputs. Returns the serialized model."""
+    # tracing runs the module: inputs go where its parameters are (only their shapes and types matter)
+    where = next((p.device for p in module.parameters()), torch.device("cpu"))
+    dummy_inputs = tuple(torch.zeros(t.shape, dtype=t.dtype, device=where) for t in dummy_inputs)
+    buf = io.BytesIO()
+    with _exporter_without_onnx_package(), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        torch.onnx.export(module, dummy_inputs, buf, opset_version=12, dynamo=False, do_constant_folding=False,
+                          keep_initializers_as_inputs=True)
+    return buf.getvalue()
+
+
 class DaceModule(nn.Module):
     """A wrapper that runs a PyTorch ``nn.Module`` on the "mi355x" expansions.
 
@@ -198,6 +244,7 @@ class DaceModule(nn.Module):
     :param backward: must be False.
     :param auto_optimize: apply the graph-level fusion pass.
     :param sdfg_name: the name to give to the SDFG (defaults to the module's class name).
+    :param exporter: "auto", "structural" or "torch": how the ONNX graph is obtained (see the module docstring).
 
     Parameters are read from ``module`` when the graph is built (first call): derived copies (k-contiguous,
     concatenated weights) are made then, so call :meth:`reset_sdfg` after changing parameters.
@@ -205,8 +252,12 @@ class DaceModule(nn.Module):
 
     def __init__(self, module: nn.Module, dummy_inputs: typing.Optional[typing.Tuple[torch.Tensor]] = None,
                  cuda: typing.Optional[bool] = None, training: bool = False, backward=False, apply_strict: bool = True,
-                 auto_optimize: bool = True, debug_transients: bool = False, sdfg_name: typing.Optional[str] = None):
+                 auto_optimize: bool = True, debug_transients: bool = False, sdfg_name: typing.Optional[str] = None,
+                 exporter: str = "auto"):
         super().__init__()
+        if exporter not in ("auto", "structural", "torch"):
+            raise ValueError(f"exporter must be 'auto', 'structural' or 'torch', got {exporter!r}")
+        self.exporter = exporter
         if backward or training:
             raise NotImplementedError("DaceModule here is inference only (backward=False, training=False)")
         if debug_transients:
@@ -231,18 +282,27 @@ class DaceModule(nn.Module):
         was_training = self.model.training
         self.model.eval()
         try:
-            self.onnx_model = module_to_onnx(self.model, dummy_inputs, name=self.sdfg_name)
+            self.onnx_model = None
+            if self.exporter != "torch":
+                try:
+                    self.onnx_model = module_to_onnx(self.model, dummy_inputs, name=self.sdfg_name)
+                except UnsupportedModule:
+                    if self.exporter == "structural":
+                        raise
+            if self.onnx_model is None:
+                from ..onnx import proto
+                self.onnx_model = proto.parse_model(export_with_torch(self.model, dummy_inputs))
         finally:
             self.model.train(was_training)
         self.dace_model = ONNXModel(self.sdfg_name, self.onnx_model, cuda=True, parent_pytorch_module=self.model,
                                     auto_optimize=self.auto_optimize)
         self.sdfg = self.dace_model.sdfg
-        self._input_shape = tuple(dummy_inputs[0].shape)
+        self._input_shapes = tuple(tuple(t.shape) for t in dummy_inputs)
 
         def forward(*args):
-            if len(args) != 1 or tuple(args[0].shape) != self._input_shape:
-                raise TypeError(f"{self.sdfg_name} was built for one input of shape {self._input_shape}")
-            return self.dace_model(args[0])
+            if tuple(tuple(a.shape) for a in args) != self._input_shapes:
+                raise TypeError(f"{self.sdfg_name} was built for inputs of shapes {self._input_shapes}")
+            return self.dace_model(*args)
 
         return forward
 

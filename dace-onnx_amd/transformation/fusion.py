@@ -687,8 +687,9 @@ def _rebase_strides(shape, strides, n_old, n_new):
 
 def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
     """MatMul nodes that multiply the same A by different constant [K, N_i] weights
-    (optionally each with a fused 1-D bias) become one MatMul against the weights
-    concatenated along N. Applies when every reader of every Y_i is a MatMul
+    (or, all of them, by [N_i, K] weights read through a folded Transpose, the form
+    ``nn.Linear`` exports to; optionally each with a fused 1-D bias) become one MatMul
+    against the weights concatenated along N. Applies when every reader of every Y_i is a MatMul
     operand, because only the GEMM can address a column slice of the wide result
     without a copy. One launch instead of len(group), and A is read once."""
     import torch
@@ -712,7 +713,7 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
     for node in state.nodes():
         if not _is_op(node, "MatMul"):
             continue
-        if any(getattr(node, a, None) is not None for a in ("_a_view", "_b_view", "_y_view", "_activation")) \
+        if any(getattr(node, a, None) is not None for a in ("_a_view", "_y_view", "_activation")) \
                 or getattr(node, "_alpha", 1.0) != 1.0 or _in_edge(state, node, "_residual") is not None:
             continue
         a_e, y_e = _in_edge(state, node, "A"), _out_edge(state, node, "Y")
@@ -720,6 +721,13 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
         if a_e is None or b_e is None or y_e is None or not isinstance(a_e.src, AccessNode) \
                 or not isinstance(y_e.dst, AccessNode):
             continue
+        # B either as ONNX stores it ([K, N]) or as nn.Linear does ([N, K] read through a folded Transpose)
+        b_view, transposed = getattr(node, "_b_view", None), False
+        if b_view is not None:
+            n_w, k_w = sdfg.arrays[b_e.src.data].shape
+            if list(b_view[0]) != [k_w, n_w] or list(b_view[1]) != [1, k_w] or (len(b_view) > 2 and b_view[2]):
+                continue
+            transposed = True
         has_bias = _in_edge(state, node, "_bias") is not None
         bias_e = constant_input(node, "_bias", 1) if has_bias else None
         if has_bias and bias_e is None:
@@ -735,21 +743,21 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
             continue
         if any(r.dst is node for r in readers):
             continue
-        k = sdfg.arrays[b_e.src.data].shape[0]
+        k, width = sdfg.arrays[b_e.src.data].shape[::-1] if transposed else sdfg.arrays[b_e.src.data].shape
         a_writes = sum(len(state.in_edges(n)) for n in state.nodes() if isinstance(n, AccessNode) and n.data == a_e.src.data)
         if a_writes > 1:
             continue
-        groups.setdefault((a_e.src.data, k, has_bias), []).append((node, a_e, b_e, bias_e, y_e, readers))
+        groups.setdefault((a_e.src.data, k, has_bias, transposed), []).append((node, a_e, b_e, bias_e, y_e, readers, width))
 
     fused = 0
-    for members in groups.values():
+    for (_, k_total, _, transposed), members in groups.items():
         if len(members) < 2:
             continue
         # a reader of one member's output must not be another member (they all run at once)
         nodes = [m[0] for m in members]
         if any(r.dst in nodes for m in members for r in m[5]):
             continue
-        widths = [sdfg.arrays[m[2].src.data].shape[1] for m in members]
+        widths = [m[6] for m in members]
         if any(w % 4 for w in widths):
             continue
         n_total = sum(widths)
@@ -760,7 +768,7 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
             continue
         # ---- new views of every reader; give up on the whole group if one cannot be expressed
         rewires, start, ok = [], 0, True
-        for (node, a_e, b_e, bias_e, y_e, readers), width in zip(members, widths):
+        for (node, a_e, b_e, bias_e, y_e, readers, _), width in zip(members, widths):
             ydesc = sdfg.arrays[y_e.dst.data]
             for r in readers:
                 attr = {"A": "_a_view", "B": "_b_view", "Q": "_q_view", "K": "_k_view", "V": "_v_view"}[r.dst_conn]
@@ -801,7 +809,8 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
             continue
         # ---- constants: weights [K, sum N_i], biases [sum N_i]
         w_name = by_clean[first[2].src.data] + "_hcat"
-        model.weights[w_name] = torch.cat([model.weights[by_clean[m[2].src.data]] for m in members], dim=1).contiguous()
+        model.weights[w_name] = torch.cat([model.weights[by_clean[m[2].src.data]] for m in members],
+                                          dim=0 if transposed else 1).contiguous()
         w_clean = clean_onnx_name(w_name)
         sdfg.add_array(w_clean, list(model.weights[w_name].shape), y0.dtype, transient=False)
         b_clean = None
@@ -817,6 +826,8 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
         keep = first[0]
         state.remove_edge(first[2])
         state.add_edge(state.add_access(w_clean), None, keep, "B", sdfg.make_array_memlet(w_clean))
+        if transposed:
+            keep._b_view = ([k_total, n_total], [1, k_total])
         if b_clean is not None:
             state.remove_edge(first[3])
             state.add_edge(state.add_access(b_clean), None, keep, "_bias", sdfg.make_array_memlet(b_clean))
@@ -826,7 +837,7 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
             state.remove_edge(r)
             state.add_edge(wide_access, None, r.dst, r.dst_conn, sdfg.make_array_memlet(wide))
             setattr(r.dst, attr, view)
-        for node, a_e, b_e, bias_e, y_e, readers in members:
+        for node, a_e, b_e, bias_e, y_e, readers, _ in members:
             if node is not keep:
                 state.remove_node(node)
             state.remove_node(y_e.dst)

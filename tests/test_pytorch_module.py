@@ -96,3 +96,69 @@ def test_conv_relu_linear_module_and_decorator():
         ref2 = copy.deepcopy(net.model).double()(x.double())
     net.reset_sdfg()
     assert rel_err(ref2.numpy(), net(x.cuda()).cpu().numpy()) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- the TorchScript exporter path
+class _TwoInputNet(nn.Module):
+    """Not a Sequential and with two inputs: only the exporter can turn it into a graph."""
+    def __init__(self):
+        super().__init__()
+        self.conv = nn.Conv2d(3, 8, 3, padding=1)
+        self.fc = nn.Linear(8 * 8 * 8, 12)
+
+    def forward(self, x, y):
+        h = torch.relu(self.conv(x)) + y
+        return torch.softmax(self.fc(h.flatten(1)), dim=-1)
+
+
+def test_exporter_path_writes_the_reference_flavoured_graph():
+    from dace_onnx_amd.onnx import proto
+    from dace_onnx_amd.pytorch.module import export_with_torch
+    layer = _bert_layer(128, 2, 256)
+    m = proto.parse_model(export_with_torch(layer, (torch.randn(2, 128, 128), )))
+    ops = {n.op_type for n in m.graph.node}
+    # no constant folding by the exporter: shape arithmetic and weight transposes are nodes
+    assert {"Unsqueeze", "Concat", "Constant", "Transpose", "MatMul", "Erf", "ReduceMean"} <= ops
+    names = {t.name for t in m.graph.initializer}
+    assert {"attention.self.query.weight", "output.dense.weight", "output.LayerNorm.bias"} <= names
+    assert names <= {i.name for i in m.graph.input}          # keep_initializers_as_inputs
+    # imported with constant folding, fused: the same seven launches as the structural graph, and the three
+    # [N, K] projection weights concatenated along N without a transposed copy
+    dm = DaceModule(layer, dummy_inputs=(torch.randn(2, 128, 128), ), exporter="torch")
+    assert sorted(_functions(dm)) == ["mi355x_attention_f32"] + ["mi355x_gemm_f32"] * 4 + ["mi355x_layernorm_f32"] * 2
+    assert tuple(dm.dace_model.weights["attention.self.query.weight_hcat"].shape) == (3 * 128, 128)
+    assert not any(k.endswith("_kcontig") for k in dm.dace_model.weights)
+    with pytest.raises(ValueError, match="exporter must be"):
+        DaceModule(layer, exporter="onnxruntime")
+
+
+def test_auto_falls_back_to_the_exporter():
+    net = _TwoInputNet().eval()
+    with pytest.raises(UnsupportedModule):
+        DaceModule(net, dummy_inputs=(torch.randn(2, 3, 8, 8), torch.randn(2, 8, 8, 8)), exporter="structural")
+    dm = DaceModule(net, dummy_inputs=(torch.randn(2, 3, 8, 8), torch.randn(2, 8, 8, 8)))
+    assert len(dm.dace_model.inputs) == 2
+    assert _functions(dm) == ["mi355x_conv2d_f32", "mi355x_eltwise_f32", "mi355x_gemm_f32", "mi355x_softmax_f32"]
+
+
+@pytest.mark.gpu
+def test_exporter_path_results():
+    torch.manual_seed(3)
+    net = _TwoInputNet().eval()
+    x, y = torch.randn(4, 3, 8, 8), torch.randn(4, 8, 8, 8)
+    with torch.no_grad():
+        ref = copy.deepcopy(net).double()(x.double(), y.double())
+    got = DaceModule(net)(x.cuda(), y.cuda())
+    assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL
+
+    layer = _bert_layer(128, 2, 256)
+    with torch.no_grad():
+        for p in layer.parameters():      # the default initialisation leaves biases at zero
+            p.add_(torch.randn_like(p) * 0.02)
+    h = torch.randn(3, 128, 128)
+    with torch.no_grad():
+        ref = copy.deepcopy(layer).double()(h.double())
+        ref = ref[0] if isinstance(ref, (tuple, list)) else ref
+    for exporter in ("torch", "structural"):
+        got = DaceModule(layer, exporter=exporter)(h.cuda())
+        assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL, exporter
