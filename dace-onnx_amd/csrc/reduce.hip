@@ -42,14 +42,15 @@ __global__ __launch_bounds__(256) void reduce_mean_strided(const float* __restri
     if (idx >= outer * inner) return;
     const int64_t o = idx / inner, i = idx % inner;
     const float* x = X + o * axis_len * inner + i;
-    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // independent chains, pairwise combination
+    // independent chains for the loads; in double, because one thread adds up a whole column
+    double s[8] = {0., 0., 0., 0., 0., 0., 0., 0.};
     int64_t a = 0;
     for (; a + 8 <= axis_len; a += 8) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s[u] += x[(a + u) * inner];
+        for (int u = 0; u < 8; ++u) s[u] += (double)x[(a + u) * inner];
     }
-    for (int u = 0; a < axis_len; ++a, ++u) s[u] += x[a * inner];
-    Y[idx] = ((((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7])))) * inv_n;
+    for (int u = 0; a < axis_len; ++a, ++u) s[u] += (double)x[a * inner];
+    Y[idx] = (float)((((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]))) / (double)axis_len);
 }
 
 }  // namespace mi355x
