@@ -225,6 +225,52 @@ def _fold_into_contractions(sdfg: SDFG, state: SDFGState) -> int:
     return folded
 
 
+def _fold_operand_scale(sdfg: SDFG, state: SDFGState) -> int:
+    """``Mul`` / ``Div`` of a MatMul operand by a scalar constant (``nn.MultiheadAttention`` scales the
+    queries before ``Q K^T``) moves into the node's alpha: (c A) B = c (A B). The scaled tensor must have
+    the MatMul as its only reader."""
+    folded = 0
+    changed = True
+    while changed:
+        changed = False
+        for node in state.nodes():
+            if not _is_op(node, "MatMul"):
+                continue
+            for conn in ("A", "B"):
+                e = _in_edge(state, node, conn)
+                if e is None or not isinstance(e.src, AccessNode) or _single_consumer(sdfg, state, e.src) is None:
+                    continue
+                prod = _producer(state, e.src)
+                if prod is None or not _is_op(prod.src, "Mul", "Div"):
+                    continue
+                scale = prod.src
+                # the constant may be either factor of a Mul, only the divisor of a Div
+                for c_conn, x_conn in (("B", "A"), ("A", "B")) if _is_op(scale, "Mul") else (("B", "A"), ):
+                    c_e, x_e = _in_edge(state, scale, c_conn), _in_edge(state, scale, x_conn)
+                    if c_e is None or x_e is None or not isinstance(x_e.src, AccessNode):
+                        continue
+                    val = _constant_value(sdfg, c_e.src.data)
+                    if val is None or val.size != 1 or \
+                            tuple(sdfg.arrays[x_e.src.data].shape) != tuple(sdfg.arrays[e.src.data].shape):
+                        continue
+                    v = float(val.reshape(-1)[0])
+                    node._alpha = getattr(node, "_alpha", 1.0) * ((1.0 / v) if _is_op(scale, "Div") else v)
+                    mid = e.src
+                    state.remove_edge(e)
+                    state.add_edge(x_e.src, None, node, conn, sdfg.make_array_memlet(x_e.src.data))
+                    state.remove_node(scale)
+                    state.remove_node(mid)
+                    del sdfg.arrays[mid.data]
+                    folded += 1
+                    changed = True
+                    break
+                if changed:
+                    break
+            if changed:
+                break
+    return folded
+
+
 # ----------------------------------------------------------------------------- view folds
 def _input_view(sdfg, state, access: AccessNode):
     """Walk back through Reshape/Transpose producers of ``access``. Returns
@@ -879,6 +925,7 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
         total += _fuse_decomposed_layernorm(sdfg, state)
         total += _fuse_decomposed_gelu(sdfg, state)
         total += _fold_into_contractions(sdfg, state)
+        total += _fold_operand_scale(sdfg, state)
         total += _fold_views(sdfg, state)
         _remove_dead_nodes(sdfg, state)  # folded Reshape/Transpose chains must not count as readers
         total += _fuse_attention(sdfg, state)

@@ -168,3 +168,23 @@ def test_rebase_and_reshape_strides():
     v = a.transpose(1, 0, 2)
     assert _reshape_strides(list(v.shape), [s // 8 for s in v.strides], [3, 8]) is None  # numpy would copy
     assert _reshape_strides([2, 3, 4], [12, 4, 1], [6, 4]) == [4, 1]
+
+
+def test_scalar_scale_on_an_operand_becomes_alpha():
+    T = proto.TensorProto
+    def model(op, const_first):
+        ins = ["c", "q"] if const_first else ["q", "c"]
+        nodes = [H.make_node(op, ins, ["qs"]), H.make_node("Transpose", ["k"], ["kt"], perm=[0, 2, 1]),
+                 H.make_node("MatMul", ["qs", "kt"], ["y"])]
+        g = H.make_graph(nodes, "g", [H.make_tensor_value_info("q", T.FLOAT, [3, 8, 16]),
+                                      H.make_tensor_value_info("k", T.FLOAT, [3, 12, 16])],
+                         [H.make_tensor_value_info("y", T.FLOAT, [3, 8, 12])],
+                         initializer=[proto.numpy_helper.from_array(np.array(0.25, np.float32), name="c")])
+        return donnx.ONNXModel("scaled_" + op + str(const_first), H.make_model(g, opset_imports=[H.make_opsetid("", 12)]))
+
+    for op, const_first, alpha in (("Mul", False, 0.25), ("Mul", True, 0.25), ("Div", False, 4.0)):
+        calls = _launches(model(op, const_first))
+        assert [f for f, _ in calls] == ["mi355x_gemm_f32"], (op, const_first)
+        assert alpha in calls[0][1]
+    # a constant numerator is not a scale of the operand: c / q stays an elementwise launch
+    assert [f for f, _ in _launches(model("Div", True))] == ["mi355x_eltwise_f32", "mi355x_gemm_f32"]

@@ -162,3 +162,32 @@ def test_exporter_path_results():
     for exporter in ("torch", "structural"):
         got = DaceModule(layer, exporter=exporter)(h.cuda())
         assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL, exporter
+
+
+def test_multihead_attention_launch_list():
+    # the module of the reference's tests/pytorch/test_attn.py, small: the exporter's 76 nodes (Shape, Gather,
+    # Slice of the packed in_proj_weight, Unsqueeze, Concat ...) fold to MatMul / Transpose / Reshape / Mul /
+    # Softmax / ReduceMean; the query scale moves into the GEMM's alpha, the transposes into operand strides
+    mha = nn.MultiheadAttention(256, 4, bias=False).eval()
+    q, k, v = torch.randn(128, 2, 256), torch.randn(128, 2, 256), torch.randn(128, 2, 256)
+    dm = DaceModule(mha, dummy_inputs=(q, k, v))
+    assert dm.dace_model.inputs == ["query", "key", "value"] and len(dm.dace_model.outputs) == 2
+    assert _functions(dm) == ["mi355x_gemm_f32"] * 4 + ["mi355x_softmax_f32"] + ["mi355x_gemm_f32"] * 2 + \
+        ["mi355x_reduce_mean_f32"]
+
+
+@pytest.mark.gpu
+def test_multihead_attention_module():
+    # tests/pytorch/test_attn.py at its own sizes: B=2, 16 heads of 64, 512 queries and keys, both outputs
+    torch.manual_seed(4)
+    B, H, P, S = 2, 16, 64, 512
+    N = P * H
+    k, q, v = torch.randn(S, B, N), torch.randn(S, B, N), torch.randn(S, B, N)
+    mha = nn.MultiheadAttention(N, H, bias=False).eval()
+    with torch.no_grad():
+        ref_out, ref_weights = copy.deepcopy(mha).double()(q.double(), k.double(), v.double())
+    out, weights = DaceModule(mha)(q.cuda(), k.cuda(), v.cuda())
+    torch_tensors_close("outputs_0", ref_out.float(), out.cpu(), rtol=1e-4, atol=1e-5)
+    torch_tensors_close("outputs_1", ref_weights.float(), weights.cpu(), rtol=1e-4, atol=1e-6)
+    assert rel_err(ref_out.numpy(), out.cpu().numpy()) < FP32_REL_TOL
+    assert rel_err(ref_weights.numpy(), weights.cpu().numpy()) < FP32_REL_TOL
