@@ -66,7 +66,8 @@ class ONNXModel:
                  fold_constants: bool = True,
                  parent_pytorch_module: typing.Optional[torch.nn.Module] = None,
                  fuse: bool = True,
-                 use_hip_graph: bool = False):
+                 use_hip_graph: bool = False,
+                 save_transients: typing.Optional[typing.Dict[str, torch.Tensor]] = None):
         """
         :param name: the name for the SDFG.
         :param model: the model to import.
@@ -80,6 +81,10 @@ class ONNXModel:
                                       module are taken from it rather than from the ONNX graph.
         :param fuse: with ``auto_optimize``, fold bias/activation/residual/transposes into contractions.
         :param use_hip_graph: replay the launch sequence as one HIP graph from the second call on.
+        :param save_transients: if not None, every intermediate value of the graph is kept and stored in
+                                this dict under its array name on each call (for debugging; as in the
+                                reference, ``onnx_importer.py:454-478``, the intermediates stop being
+                                transients, so nothing is fused across them).
         """
         if not isinstance(model, ModelProto):
             model = proto.load(model)
@@ -90,6 +95,9 @@ class ONNXModel:
         self.do_auto_optimize = auto_optimize
         self.fuse = fuse
         self.use_hip_graph = use_hip_graph
+        self.save_transients = save_transients
+        if save_transients is not None and use_hip_graph:
+            raise ValueError("save_transients allocates fresh tensors on every call: not with use_hip_graph")
         model = self._constants_to_initializers(model)
         if fold_constants:
             from ..transformation.constant_folding import fold_constants as _fold
@@ -279,6 +287,10 @@ class ONNXModel:
         """Apply the graph-level fusion (if enabled) and expand every ONNX node to kernel
         calls; returns the SDFG. Needs no GPU."""
         if not self._expanded:
+            if self.save_transients is not None:
+                self._saved = [k for k, d in self.sdfg.arrays.items() if d.transient]
+                for k in self._saved:
+                    self.sdfg.arrays[k].transient = False
             if self.do_auto_optimize:
                 self.auto_optimize()
             from ..util.utils import expand_onnx_nodes
@@ -353,6 +365,11 @@ class ONNXModel:
                 desc = self.sdfg.arrays[clean_onnx_name(n)]
                 outputs[n] = torch.empty(desc.shape, dtype=desc.dtype.as_torch(), device=self.device)
             out_kwargs = {clean_onnx_name(n): t for n, t in outputs.items()}
+            if self.save_transients is not None:
+                for k in self._saved:
+                    desc = self.sdfg.arrays[k]
+                    out_kwargs[k] = self.save_transients[k] = torch.empty(desc.shape, dtype=desc.dtype.as_torch(),
+                                                                          device=self.device)
             compiled(**call, **out_kwargs, **self.clean_weights)
         results = [t if use_torch else t.cpu().numpy() for t in outputs.values()]
         return results[0] if len(results) == 1 else tuple(results)

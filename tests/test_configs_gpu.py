@@ -290,3 +290,28 @@ def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
     if epi & 8:
         ref = ref + res.double()
     assert rel_err(ref.cpu().numpy(), out.cpu().numpy()) < FP32_REL_TOL
+
+
+def test_save_transients_keeps_every_intermediate(golden):
+    # the reference's ONNXModel(save_transients=...) (tests/test_bert_subgraphs.py:37-52): intermediates are
+    # kept, so the graph runs node by node; each saved tensor is checked against the oracle's value
+    hidden, heads, ffn, bsz, seq = (int(v) for v in golden["bert_meta"])
+    w = {k[len("bert_"):]: golden[k] for k in golden.files if k.startswith("bert_") and k not in
+         ("bert_x", "bert_y", "bert_meta")}
+    saved = {}
+    model = donnx.ONNXModel("bert_saved", bert_encoder_layer_model(w, bsz, seq, heads), save_transients=saved)
+    got = model(golden["bert_x"])
+    assert rel_err(golden["bert_y"], got) < FP32_REL_TOL
+    assert model.compile_and_init().num_launches == 26        # nothing was fused away
+    x = golden["bert_x"]
+    d = hidden // heads
+    q = O.add(O.matmul(x, w["wq"]), w["bq"])
+    q_heads = O.transpose(O.reshape(q, (bsz, seq, heads, d)), (0, 2, 1, 3))
+    k_heads = O.transpose(O.reshape(O.add(O.matmul(x, w["wk"]), w["bk"]), (bsz, seq, heads, d)), (0, 2, 1, 3))
+    probs = O.softmax(O.matmul(q_heads, O.transpose(k_heads, (0, 1, 3, 2))) / np.float32(np.sqrt(d)), axis=3)
+    for name, expected in (("q_lin", q), ("q_heads", q_heads), ("probs", probs)):
+        assert rel_err(expected, saved[name].cpu().numpy()) < FP32_REL_TOL, name
+    assert {"attn_res", "h1", "inter", "ffn_res", "ctx"} <= set(saved) and "y" not in saved
+    with pytest.raises(ValueError, match="not with use_hip_graph"):
+        donnx.ONNXModel("bert_saved_graph", bert_encoder_layer_model(w, bsz, seq, heads), save_transients={},
+                        use_hip_graph=True)
