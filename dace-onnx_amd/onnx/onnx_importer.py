@@ -298,6 +298,13 @@ class ONNXModel:
             self._expanded = True
         return self.sdfg
 
+    def expand_onnx_nodes(self):
+        """Expand every ONNX node of the SDFG as it is (no fusion); the reference's method of the same
+        name (``onnx_importer.py:574-575``). :meth:`expand` is the fusing variant ``__call__`` uses."""
+        from ..util.utils import expand_onnx_nodes
+        expand_onnx_nodes(self.sdfg)
+        self._expanded = True
+
     def compile_and_init(self):
         if self._compiled is None:
             if self.device.type != "cuda":
@@ -373,3 +380,16 @@ class ONNXModel:
             compiled(**call, **out_kwargs, **self.clean_weights)
         results = [t if use_torch else t.cpu().numpy() for t in outputs.values()]
         return results[0] if len(results) == 1 else tuple(results)
+
+
+def create_output_array(inferred_symbols: typing.Dict[str, int], desc, use_torch: bool = False, zeros: bool = False):
+    """The array for an output described by ``desc`` (``onnx_importer.py:586-633`` in the reference): a torch
+    tensor on the GPU when ``use_torch``. Outputs live in device memory here, so ``use_torch=False`` is refused
+    like the reference refuses a GPU descriptor without it. ``inferred_symbols`` is accepted for signature
+    compatibility: shapes are static."""
+    if not use_torch:
+        raise ValueError("Got use_torch=False, but received a GPU descriptor")
+    shape = [int(d) for d in desc.shape]
+    make = torch.zeros if zeros else torch.empty
+    device = torch.device("cuda:0" if torch.cuda.is_available() else "cpu")
+    return make(shape if shape else [1], dtype=desc.dtype.as_torch(), device=device).reshape(shape)

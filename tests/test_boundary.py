@@ -7,6 +7,7 @@ import re
 
 import numpy as np
 import pytest
+import torch
 
 import dace_onnx_amd as dml
 from dace_onnx_amd import _lib, sdfg as dace
@@ -318,3 +319,20 @@ def test_daceml_adapter_mirrors_nodes_and_needs_the_real_packages():
     assert daceml_adapter.mirror_expansion(mm, st, sdfg) is None
     with pytest.raises(ImportError, match="dace"):
         daceml_adapter.register()
+
+
+def test_onnx_model_helpers_of_the_reference_api():
+    # ONNXModel.expand_onnx_nodes (expansion without fusion) and create_output_array (onnx_importer.py:574-633)
+    from dace_onnx_amd.onnx.onnx_importer import create_output_array
+    from dace_onnx_amd.testing.graphs import conv_relu_model
+    rng = np.random.default_rng(0)
+    m = conv_relu_model(rng.normal(size=(4, 3, 3, 3)).astype(np.float32), np.zeros(4, np.float32), (1, 3, 8, 8))
+    model = donnx.ONNXModel("conv_relu_unfused", m)
+    model.expand_onnx_nodes()
+    fns = [n.function for n, _ in model.sdfg.all_nodes_recursive() if isinstance(n, dace.KernelCall)]
+    assert fns == ["mi355x_conv2d_f32", "mi355x_eltwise_f32"]      # Relu not folded into the convolution
+    desc = model.sdfg.arrays["Y"]
+    out = create_output_array({}, desc, use_torch=True, zeros=True)
+    assert tuple(out.shape) == tuple(desc.shape) and out.dtype == torch.float32 and float(out.abs().sum()) == 0.0
+    with pytest.raises(ValueError, match="use_torch=False"):
+        create_output_array({}, desc, use_torch=False)
