@@ -27,8 +27,10 @@ Two ways to the graph here (``exporter=``):
 Inference only: ``backward=True`` is refused (the reference's autodiff is a separate
 subsystem).
 """
+import collections
 import contextlib
 import io
+import logging
 import math
 import typing
 import warnings
@@ -40,6 +42,9 @@ import torch.nn as nn
 
 from ..onnx.onnx_importer import ONNXModel
 from ..onnx.proto import helper, numpy_helper, TensorProto, ModelProto
+
+
+log = logging.getLogger(__name__)
 
 
 class UnsupportedModule(NotImplementedError):
@@ -242,7 +247,9 @@ class DaceModule(nn.Module):
     :param cuda: kept for signature compatibility: execution is always on the GPU.
     :param training: must be False (the graph is the inference graph).
     :param backward: must be False.
-    :param auto_optimize: apply the graph-level fusion pass.
+    :param auto_optimize: apply the graph-level fusion pass (registered as the post-ONNX hook "auto_optimize").
+    :param debug_transients: every intermediate value becomes an additional output of the module (a post-ONNX
+                             hook placed before the optimisation, so nothing is fused across them).
     :param sdfg_name: the name to give to the SDFG (defaults to the module's class name).
     :param exporter: "auto", "structural" or "torch": how the ONNX graph is obtained (see the module docstring).
 
@@ -260,8 +267,6 @@ class DaceModule(nn.Module):
         self.exporter = exporter
         if backward or training:
             raise NotImplementedError("DaceModule here is inference only (backward=False, training=False)")
-        if debug_transients:
-            raise NotImplementedError("debug_transients is not supported")
         self.model = module
         self.dace_model: typing.Optional[ONNXModel] = None
         self.onnx_model: typing.Optional[ModelProto] = None
@@ -269,7 +274,29 @@ class DaceModule(nn.Module):
         self.use_cuda = True
         self.sdfg_name = sdfg_name or type(module).__name__
         self.auto_optimize = auto_optimize
+        self.debug_transients = debug_transients
         self.function = None
+        #: hooks executed after the ONNX graph is imported to an SDFG, each called with this module
+        self.post_onnx_hooks: "collections.OrderedDict[str, typing.Callable]" = collections.OrderedDict()
+        #: hooks executed after the SDFG is compiled, each called with the compiled SDFG
+        self.post_compile_hooks: "collections.OrderedDict[str, typing.Callable]" = collections.OrderedDict()
+
+        # the reference's own use of its hooks (daceml/pytorch/module.py:98-146): the debugging option first,
+        # the optimisation pass last, so that user hooks appended later run on the optimised graph
+        if debug_transients:
+            def transients_outputs(dace_module):
+                model = dace_module.dace_model
+                for name, desc in model.sdfg.arrays.items():
+                    if desc.transient:
+                        desc.transient = False
+                        model.outputs.append(name)
+            self.prepend_post_onnx_hook("make_transients_outputs", transients_outputs)
+        if auto_optimize:
+            def auto_optimize_hook(dace_module):
+                from ..util import utils
+                utils.auto_optimize(dace_module.dace_model.sdfg, cuda=True)
+                dace_module.dace_model._expanded = True
+            self.append_post_onnx_hook("auto_optimize", auto_optimize_hook)
         if dummy_inputs is not None:
             self.function = self._initialize_sdfg(dummy_inputs)
 
@@ -277,6 +304,35 @@ class DaceModule(nn.Module):
         """Drop the compiled graph; the next call rebuilds it from the module's current parameters."""
         self.function = None
         self.dace_model = self.onnx_model = self.sdfg = None
+
+    @staticmethod
+    def _unique(existing, name):
+        candidate, i = name, 0
+        while candidate in existing:
+            i += 1
+            candidate = f"{name}_{i}"
+        return candidate
+
+    def _add_hook(self, hooks, name, func, first):
+        if self.function is not None:
+            log.warning("Added a hook after the model was already initialized. This hook will not be executed "
+                        "until reset_sdfg() is called.")
+        name = self._unique(hooks, name)
+        hooks[name] = func
+        if first:
+            hooks.move_to_end(name, last=False)
+
+    def prepend_post_onnx_hook(self, name: str, func: typing.Callable[["DaceModule"], None]):
+        self._add_hook(self.post_onnx_hooks, name, func, first=True)
+
+    def append_post_onnx_hook(self, name: str, func: typing.Callable[["DaceModule"], None]):
+        self._add_hook(self.post_onnx_hooks, name, func, first=False)
+
+    def prepend_post_compile_hook(self, name: str, func: typing.Callable):
+        self._add_hook(self.post_compile_hooks, name, func, first=True)
+
+    def append_post_compile_hook(self, name: str, func: typing.Callable):
+        self._add_hook(self.post_compile_hooks, name, func, first=False)
 
     def _initialize_sdfg(self, dummy_inputs):
         was_training = self.model.training
@@ -294,14 +350,22 @@ class DaceModule(nn.Module):
                 self.onnx_model = proto.parse_model(export_with_torch(self.model, dummy_inputs))
         finally:
             self.model.train(was_training)
+        # optimisation is a hook of this module, not of the ONNXModel (which would apply it on its first call)
         self.dace_model = ONNXModel(self.sdfg_name, self.onnx_model, cuda=True, parent_pytorch_module=self.model,
-                                    auto_optimize=self.auto_optimize)
+                                    auto_optimize=False)
         self.sdfg = self.dace_model.sdfg
+        for hook in self.post_onnx_hooks.values():
+            hook(self)
         self._input_shapes = tuple(tuple(t.shape) for t in dummy_inputs)
+        state = {"compiled": None}
 
         def forward(*args):
             if tuple(tuple(a.shape) for a in args) != self._input_shapes:
                 raise TypeError(f"{self.sdfg_name} was built for inputs of shapes {self._input_shapes}")
+            if state["compiled"] is None:     # needs the GPU: done on the first call, not at construction
+                state["compiled"] = self.dace_model.compile_and_init()
+                for hook in self.post_compile_hooks.values():
+                    hook(state["compiled"])
             return self.dace_model(*args)
 
         return forward

@@ -191,3 +191,42 @@ def test_multihead_attention_module():
     torch_tensors_close("outputs_1", ref_weights.float(), weights.cpu(), rtol=1e-4, atol=1e-6)
     assert rel_err(ref_out.numpy(), out.cpu().numpy()) < FP32_REL_TOL
     assert rel_err(ref_weights.numpy(), weights.cpu().numpy()) < FP32_REL_TOL
+
+
+def test_hooks_run_in_order_and_can_change_the_graph():
+    # daceml/pytorch/module.py:83-210: named hooks after the ONNX import and after compilation
+    m = nn.Sequential(nn.Linear(8, 16), nn.ReLU(), nn.Linear(16, 4)).eval()
+    seen = []
+    dm = DaceModule(m)
+    assert list(dm.post_onnx_hooks) == ["auto_optimize"]
+    dm.append_post_onnx_hook("after", lambda mod: seen.append(("after", len(_functions(mod)))))
+    dm.prepend_post_onnx_hook("before", lambda mod: seen.append(
+        ("before", sorted(type(n).__name__ for n in mod.sdfg.states()[0].nodes() if type(n).__name__.startswith("ONNX")))))
+    dm.append_post_onnx_hook("after", lambda mod: seen.append(("after_1", None)))      # same name: made unique
+    assert list(dm.post_onnx_hooks) == ["before", "auto_optimize", "after", "after_1"]
+    dm.function = dm._initialize_sdfg((torch.randn(5, 8), ))
+    # "before" saw the imported ONNX nodes, "after" the fused and expanded graph: two GEMM launches
+    assert seen == [("before", ["ONNXGemm", "ONNXGemm", "ONNXRelu"]), ("after", 2), ("after_1", None)]
+    # without the optimisation hook the graph is expanded node by node on the first call
+    plain = DaceModule(m, dummy_inputs=(torch.randn(5, 8), ), auto_optimize=False)
+    assert list(plain.post_onnx_hooks) == [] and not plain.dace_model._expanded
+
+
+@pytest.mark.gpu
+def test_debug_transients_and_compile_hook():
+    torch.manual_seed(5)
+    m = nn.Sequential(nn.Linear(8, 16), nn.ReLU(), nn.Linear(16, 4)).eval()
+    x = torch.randn(5, 8)
+    compiled = []
+    dm = DaceModule(m, debug_transients=True)
+    dm.append_post_compile_hook("record", compiled.append)
+    outs = dm(x.cuda())
+    # the module's output first, then every intermediate (here: the two values between the three nodes)
+    assert isinstance(outs, tuple) and len(outs) == 3 and len(compiled) == 1 and compiled[0].num_launches == 3
+    with torch.no_grad():
+        h = m[0](x)
+        expected = [m(x), h, torch.relu(h)]
+    for got, ref in zip(outs, expected):
+        assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL
+    dm(x.cuda())
+    assert len(compiled) == 1          # compiled once
