@@ -1,5 +1,6 @@
 // Fused scaled-dot-product attention core, fp32:  O = softmax(scale * Q K^T) V
-// for one (batch, head) per slice, keys = 128, head size = 64 (BERT-base).
+// for one (batch, head) per slice, head size = 64; 128 keys (BERT-base) in one pass, any other number of
+// keys in blocks of 128 with a running maximum and sum.
 //
 // The reference runs this as three library nodes -- MatMul, Softmax, MatMul
 // (daceml/onnx/op_implementations/pure_implementations.py:130-235, 346-366) -- with
@@ -29,7 +30,7 @@ constexpr int AT_SK = 128, AT_D = 64, AT_BQ = 64, AT_PITCH = AT_D + LDS_PAD;
 
 struct AttnArgs {
     const float* Q; const float* K; const float* V; float* O;
-    int64_t batch1, Sq, q_blocks, nwg;
+    int64_t batch1, Sq, Sk, q_blocks, nwg;
     int64_t q_sb0, q_sb1, q_sr, k_sb0, k_sb1, k_sr, v_sb0, v_sb1, v_sr, o_sb0, o_sb1, o_sr;
     float scale;
 };
@@ -155,6 +156,133 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p) {
     }
 }
 
+// Any number of keys: the same workgroup walks the keys in blocks of 128 with a running row maximum and
+// row sum (the probabilities of a block are exp(s - running max); when the maximum grows, the sums and the
+// output accumulators are rescaled by exp(old max - new max); the division by the row sum happens once, at
+// the end). Keys beyond Sk in the last block are loaded from the last valid row and their scores set to
+// -inf. Every wave takes part in the barriers of every block, so there is no early exit for query rows
+// beyond Sq: they are computed on the clamped last row and not stored.
+__global__ __launch_bounds__(256) void attention_f32_blocks_kernel(AttnArgs p) {
+    constexpr int SK = AT_SK, D = AT_D, PITCH = AT_PITCH, NJ = SK / 16, NC = D / 16;
+    __shared__ __attribute__((aligned(16))) float lds_k[SK * PITCH];
+    __shared__ __attribute__((aligned(16))) float lds_v[SK * PITCH];
+
+    const int tid = threadIdx.x;
+    const int lane = tid % WAVE, wave = tid / WAVE;
+    const int li = lane % 16, lq = lane / 16;
+
+    const int64_t logical = xcd_remap(blockIdx.x, p.nwg);
+    const int64_t slice = logical / p.q_blocks, qb = logical % p.q_blocks;
+    const int64_t b0 = slice / p.batch1, b1 = slice % p.batch1;
+    const float* __restrict__ Q = p.Q + b0 * p.q_sb0 + b1 * p.q_sb1;
+    const float* __restrict__ K = p.K + b0 * p.k_sb0 + b1 * p.k_sb1;
+    const float* __restrict__ V = p.V + b0 * p.v_sb0 + b1 * p.v_sb1;
+    float* __restrict__ O = p.O + b0 * p.o_sb0 + b1 * p.o_sb1;
+    const int64_t q0 = qb * AT_BQ + 16 * wave;   // first query row of this wave
+
+    f32x4 rq[NC];
+    {
+        int64_t qrow = q0 + li;
+        qrow = qrow < p.Sq ? qrow : p.Sq - 1;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) rq[c] = *reinterpret_cast<const f32x4*>(Q + qrow * p.q_sr + 16 * c + 4 * lq);
+    }
+    f32x4 out[4];                       // out[t][r] = O[q0 + 4 lq + r][4 li + t], not yet divided by the row sum
+#pragma unroll
+    for (int t = 0; t < 4; ++t) out[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;   // of query row q0 + li (the same value in its four lanes)
+
+    for (int64_t key0 = 0; key0 < p.Sk; key0 += SK) {
+        f32x4 rk[8], rv[8];
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int idx = tid + it * 256, c4 = idx % (D / 4);
+            int64_t row = key0 + idx / (D / 4);
+            row = row < p.Sk ? row : p.Sk - 1;
+            rk[it] = *reinterpret_cast<const f32x4*>(K + row * p.k_sr + 4 * c4);
+            rv[it] = *reinterpret_cast<const f32x4*>(V + row * p.v_sr + 4 * c4);
+        }
+        if (key0 > 0) __syncthreads();   // the previous block's operands have been read by everyone
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int idx = tid + it * 256, row = idx / (D / 4), c4 = idx % (D / 4);
+            *reinterpret_cast<f32x4*>(lds_k + row * PITCH + 4 * c4) = rk[it];
+            *reinterpret_cast<f32x4*>(lds_v + row * PITCH + 4 * c4) = rv[it];
+        }
+        __syncthreads();
+
+        // ---- S = Q K^T of this block: acc[j][r] = S[q0 + li][key0 + 16 j + 4 lq + r]
+        f32x4 acc[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            f32x4 kf[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                kf[j] = *reinterpret_cast<const f32x4*>(lds_k + (16 * j + li) * PITCH + 16 * c + 4 * lq);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[j][s], rq[c][s], acc[j], 0, 0, 0);
+        }
+        const bool ragged = key0 + SK > p.Sk;   // uniform
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            acc[j] *= p.scale;
+            if (ragged) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (key0 + 16 * j + 4 * lq + r >= p.Sk) acc[j][r] = -INFINITY;
+            }
+            m_blk = fmaxf(m_blk, fmaxf(fmaxf(acc[j].x, acc[j].y), fmaxf(acc[j].z, acc[j].w)));
+        }
+        const float m_new = fmaxf(m_run, quad_lanes_max(m_blk));
+        const float alpha = expf(m_run - m_new);    // 0 for the first block
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            acc[j].x = expf(acc[j].x - m_new);
+            acc[j].y = expf(acc[j].y - m_new);
+            acc[j].z = expf(acc[j].z - m_new);
+            acc[j].w = expf(acc[j].w - m_new);
+            sum += (acc[j].x + acc[j].y) + (acc[j].z + acc[j].w);
+        }
+        l_run = l_run * alpha + quad_lanes_sum(sum);
+        m_run = m_new;
+        // the accumulators hold rows 4 lq + r: that row's factor lives in lane 4 lq + r
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float a = __shfl(alpha, 4 * lq + r, WAVE);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) out[t][r] *= a;
+        }
+        // ---- out += P V of this block
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            f32x4 vf[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                vf[r] = *reinterpret_cast<const f32x4*>(lds_v + (16 * j + 4 * lq + r) * PITCH + 4 * li);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    out[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(acc[j][r], vf[r][t], out[t], 0, 0, 0);
+        }
+    }
+    const float inv = 1.0f / l_run;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const float a = __shfl(inv, 4 * lq + r, WAVE);
+        const int64_t qrow = q0 + 4 * lq + r;
+        if (qrow < p.Sq)
+            *reinterpret_cast<f32x4*>(O + qrow * p.o_sr + 4 * li) = f32x4{out[0][r] * a, out[1][r] * a, out[2][r] * a, out[3][r] * a};
+    }
+}
+
 }  // namespace mi355x
 
 extern "C" int mi355x_attention_f32(const float* Q, const float* K, const float* V, float* O,
@@ -164,7 +292,7 @@ extern "C" int mi355x_attention_f32(const float* Q, const float* K, const float*
                                     float scale, void* stream) {
     using namespace mi355x;
     MI355X_REQUIRE(batch0 >= 0 && batch1 >= 0 && Sq >= 0, "attention: negative extent");
-    MI355X_REQUIRE(Sk == AT_SK && D == AT_D, "attention: only 128 keys of head size 64 are supported (got %lld x %lld)",
+    MI355X_REQUIRE(Sk >= 1 && D == AT_D, "attention: head size 64 and at least one key are required (got %lld keys x %lld)",
                    (long long)Sk, (long long)D);
     if (batch0 * batch1 == 0 || Sq == 0) return MI355X_OK;
     MI355X_REQUIRE(Q && K && V && O && q_strides && k_strides && v_strides && o_strides, "attention: null pointer");
@@ -176,7 +304,7 @@ extern "C" int mi355x_attention_f32(const float* Q, const float* K, const float*
     MI355X_REQUIRE(ok, "attention: operands must be 16-byte aligned with strides that are multiples of 4 floats");
     AttnArgs p;
     p.Q = Q; p.K = K; p.V = V; p.O = O;
-    p.batch1 = batch1; p.Sq = Sq;
+    p.batch1 = batch1; p.Sq = Sq; p.Sk = Sk;
     p.q_blocks = ceil_div(Sq, (int64_t)AT_BQ);
     p.nwg = batch0 * batch1 * p.q_blocks;
     MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "attention: grid too large");
@@ -185,6 +313,10 @@ extern "C" int mi355x_attention_f32(const float* Q, const float* K, const float*
     p.v_sb0 = v_strides[0]; p.v_sb1 = v_strides[1]; p.v_sr = v_strides[2];
     p.o_sb0 = o_strides[0]; p.o_sb1 = o_strides[1]; p.o_sr = o_strides[2];
     p.scale = scale;
-    hipLaunchKernelGGL(attention_f32_kernel, dim3((unsigned)p.nwg), dim3(256), 0, static_cast<hipStream_t>(stream), p);
-    return check_launch("attention_f32_kernel");
+    if (Sk == AT_SK) {
+        hipLaunchKernelGGL(attention_f32_kernel, dim3((unsigned)p.nwg), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        return check_launch("attention_f32_kernel");
+    }
+    hipLaunchKernelGGL(attention_f32_blocks_kernel, dim3((unsigned)p.nwg), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return check_launch("attention_f32_blocks_kernel");
 }

@@ -415,7 +415,11 @@ class MI355XFusedAttention(ONNXForward):
     fusion pass attached (``_q_view`` ... ``_o_view``): head split / merge of a
     [B, S, H*D] projection is addressing, not a copy."""
 
-    SUPPORTED_KEYS, SUPPORTED_HEAD = 128, 64
+    SUPPORTED_HEAD = 64   #: head size of the kernel; 128 keys run in one pass, any other number in blocks of 128
+
+    @staticmethod
+    def supports(plan) -> bool:
+        return plan is not None and plan[3] >= 1 and plan[4] == MI355XFusedAttention.SUPPORTED_HEAD
 
     @staticmethod
     def _operands(node, state, sdfg):
@@ -452,8 +456,7 @@ class MI355XFusedAttention(ONNXForward):
     @staticmethod
     def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
         plan = MI355XFusedAttention._plan(MI355XFusedAttention._operands(node, state, sdfg))
-        return plan is not None and plan[3] == MI355XFusedAttention.SUPPORTED_KEYS and \
-            plan[4] == MI355XFusedAttention.SUPPORTED_HEAD
+        return MI355XFusedAttention.supports(plan)
 
     @staticmethod
     def forward(node, state: SDFGState, sdfg: SDFG):

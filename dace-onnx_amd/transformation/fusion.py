@@ -25,7 +25,7 @@ ReduceMean, Sub, Pow(2), ReduceMean,         LayerNormalization (what exporters 
 Add(eps), Sqrt, Div, Mul(gamma), Add(beta)   opset 17 write for ``nn.LayerNorm``)
 Div(sqrt 2), Erf, Add(1), Mul(x), Mul(0.5)   Gelu (exact erf form, any operand order)
 MatMul(alpha) -> Softmax(last) -> MatMul     FusedAttention when the kernel supports the
-                                             shape (128 keys, head size 64)
+                                             shape (head size 64)
 MatMuls of one A with constant weights       one MatMul with the weights (and biases)
 (the Q, K, V projections)                    concatenated along N; the readers
                                              address their slice of the wide result
@@ -696,7 +696,7 @@ def _fuse_attention(sdfg: SDFG, state: SDFGState) -> int:
         kv = [ktv[0][:-2] + [ktv[0][-1], ktv[0][-2]], ktv[1][:-2] + [ktv[1][-1], ktv[1][-2]], ktv[2]]  # K = (K^T)^T
         f32 = sdfg.arrays[q_e.data.data].dtype
         plan = MI355XFusedAttention._plan([(Array(f32, v[0], v[1]), v[2]) for v in (qv, kv, vv, ov)])
-        if plan is None or plan[3] != MI355XFusedAttention.SUPPORTED_KEYS or plan[4] != MI355XFusedAttention.SUPPORTED_HEAD:
+        if not MI355XFusedAttention.supports(plan):
             continue
         node = get_onnx_node("FusedAttention")(mm1.label + "_attention", scale=float(getattr(mm1, "_alpha", 1.0)))
         state.add_node(node)
@@ -837,7 +837,7 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
                 from ..onnx.op_implementations.mi355x_implementations import MI355XFusedAttention
                 cur = [views.get(a, getattr(consumer, a)) for a in ("_q_view", "_k_view", "_v_view", "_o_view")]
                 plan = MI355XFusedAttention._plan([(Array(y0.dtype, v[0], v[1]), v[2]) for v in cur])
-                if plan is None or plan[3] != MI355XFusedAttention.SUPPORTED_KEYS or plan[4] != MI355XFusedAttention.SUPPORTED_HEAD:
+                if not MI355XFusedAttention.supports(plan):
                     ok = False
                 continue
 

@@ -134,9 +134,10 @@ int mi355x_softmax_f32(const float* X, float* Y,
  * expressed without a copy. Replaces the node sequence MatMul -> (Div | Mul by a
  * scalar) -> Softmax(last axis) -> MatMul that the reference expands one node at a
  * time (pure_implementations.py:130-235, 346-366); the score tensor never reaches
- * memory. Supported: Sk == 128, D == 64; anything else returns
- * MI355X_ERR_INVALID_ARGUMENT and launches nothing (the caller keeps the three
- * separate nodes). */
+ * memory. Supported: D == 64 and any Sk >= 1 (128 keys in one pass, any other
+ * number in blocks of 128 with a running row maximum and sum); another head size
+ * returns MI355X_ERR_INVALID_ARGUMENT and launches nothing (the caller keeps the
+ * three separate nodes). */
 int mi355x_attention_f32(const float* Q, const float* K, const float* V, float* O,
                          int64_t batch0, int64_t batch1, int64_t Sq, int64_t Sk, int64_t D,
                          const int64_t* q_strides, const int64_t* k_strides,

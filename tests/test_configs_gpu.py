@@ -315,3 +315,17 @@ def test_save_transients_keeps_every_intermediate(golden):
     with pytest.raises(ValueError, match="not with use_hip_graph"):
         donnx.ONNXModel("bert_saved_graph", bert_encoder_layer_model(w, bsz, seq, heads), save_transients={},
                         use_hip_graph=True)
+
+
+@pytest.mark.parametrize("seq", [40, 200, 384])
+def test_bert_layer_other_sequence_lengths(seq):
+    # sequence lengths other than the benchmark's 128: the fused attention kernel walks the keys in blocks
+    rng = np.random.default_rng(seq)
+    w = O.bert_layer_weights(rng, hidden=256, ffn=512)
+    for k in ("bq", "bk", "bv", "bo", "b1", "b2"):
+        w[k] = rng.normal(0.0, 0.02, size=w[k].shape).astype(np.float32)
+    x = rng.normal(size=(3, seq, 256)).astype(np.float32)
+    model = donnx.ONNXModel(f"bert_seq{seq}", bert_encoder_layer_model(w, 3, seq, 4))
+    got = model(x)
+    assert model.compile_and_init().num_launches == 7
+    assert rel_err(O.bert_layer(x, w, heads=4), got) < FP32_REL_TOL

@@ -225,9 +225,29 @@ def test_fused_attention_c_abi(batch, sq):
     Q, K, V = (t.permute(0, 2, 1, 3).cpu().numpy().astype(np.float64) for t in (q, k, v))
     expected = O.matmul(O.softmax(O.matmul(Q, np.swapaxes(K, -1, -2)) * scale, axis=-1), V)
     assert rel_err(expected, out.permute(0, 2, 1, 3).cpu().numpy()) < FP32_REL_TOL
-    # unsupported shapes are rejected, nothing is launched
-    assert lib.mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq, 64, 64,
+    # another head size is rejected, nothing is launched
+    assert lib.mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq, 128, 32,
                                     strides(q), strides(k), strides(v), strides(out), scale, _lib.current_stream()) == 1
+
+
+@pytest.mark.parametrize("sk", [1, 5, 64, 127, 129, 200, 256, 384, 1000])
+def test_fused_attention_any_number_of_keys(sk):
+    # keys walked in blocks of 128 with a running row maximum and sum; the last block may be ragged.
+    # Scores with a large spread (scale 1) so that the running maximum really moves between blocks.
+    rng = np.random.default_rng(sk)
+    b0, b1, sq = 2, 3, 70
+    q = torch.from_numpy(rng.normal(size=(b0, b1, sq, 64)).astype(np.float32)).cuda()
+    k = torch.from_numpy(rng.normal(size=(b0, b1, sk, 64)).astype(np.float32)).cuda()
+    v = torch.from_numpy(rng.normal(size=(b0, b1, sk, 64)).astype(np.float32)).cuda()
+    out = torch.full((b0, b1, sq, 64), float("nan"), device="cuda")
+    strides = lambda t: _lib.i64_array([t.stride(0), t.stride(1), t.stride(2)])
+    _lib.check(_lib.library().mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq,
+                                                   sk, 64, strides(q), strides(k), strides(v), strides(out), 1.0,
+                                                   _lib.current_stream()), "mi355x_attention_f32")
+    Q, K, V = (t.cpu().numpy().astype(np.float64) for t in (q, k, v))
+    expected = O.matmul(O.softmax(O.matmul(Q, np.swapaxes(K, -1, -2)), axis=-1), V)
+    got = out.cpu().numpy()
+    assert not np.isnan(got).any() and rel_err(expected, got) < FP32_REL_TOL
 
 
 # ----------------------------------------------------------------------------- elementwise

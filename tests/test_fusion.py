@@ -62,8 +62,13 @@ def test_bert_base_attention_core_is_one_launch():
     assert a[4:9] == [2, 12, 128, 128, 64]
     assert a[9] == a[10] == a[11] == [128 * 2304, 64, 2304] and a[12] == [128 * 768, 64, 768]
     assert a[13] == pytest.approx(0.125)
-    # 64 keys: not a shape the kernel supports, the three nodes stay
-    calls = _launches(donnx.ONNXModel("bert_s64", bert_encoder_layer_model(w, 2, 64, 12)))
+    # any other number of keys fuses as well (the kernel walks them in blocks of 128) ...
+    calls = _launches(donnx.ONNXModel("bert_s200", bert_encoder_layer_model(w, 2, 200, 12)))
+    assert [f for f, _ in calls].count("mi355x_attention_f32") == 1 and len(calls) == 7
+    a = [args for f, args in calls if f == "mi355x_attention_f32"][0]
+    assert a[4:9] == [2, 12, 200, 200, 64]
+    # ... another head size does not: the three nodes stay
+    calls = _launches(donnx.ONNXModel("bert_d96", bert_encoder_layer_model(w, 2, 128, 8)))
     assert [f for f, _ in calls].count("mi355x_attention_f32") == 0 and len(calls) == 9
 
 

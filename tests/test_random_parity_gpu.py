@@ -177,14 +177,15 @@ def test_random_attention():
     for case in range(30):
         b0, b1, sq = int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(rng.choice([1, 16, 50, 64, 65, 128, 200]))
         scale = float(rng.choice([0.125, 1.0, 0.3]))
-        tag = f"attention case {case}: b{b0}x{b1} sq{sq} scale{scale}"
+        sk = int(rng.choice([128, 128, 1, 77, 130, 300, 512]))
+        tag = f"attention case {case}: b{b0}x{b1} sq{sq} sk{sk} scale{scale}"
         print(tag, flush=True)
         # Q, K, V as slices of one packed projection result, heads interleaved: the strided form the fusion produces
-        pack = torch.from_numpy(rng.normal(size=(b0, max(sq, 128), b1, 3, 64)).astype(np.float32)).to(dev)
-        q, k, v = pack[:, :sq, :, 0], pack[:, :128, :, 1], pack[:, :128, :, 2]
+        pack = torch.from_numpy(rng.normal(size=(b0, max(sq, sk), b1, 3, 64)).astype(np.float32)).to(dev)
+        q, k, v = pack[:, :sq, :, 0], pack[:, :sk, :, 1], pack[:, :sk, :, 2]
         out = torch.full((b0, sq, b1, 64), float("nan"), device=dev)
         st3 = lambda t: _lib.i64_array([t.stride(0), t.stride(2), t.stride(1)])
-        st = lib.mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq, 128, 64,
+        st = lib.mi355x_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), b0, b1, sq, sk, 64,
                                       st3(q), st3(k), st3(v), st3(out), scale, stream())
         torch.cuda.synchronize()
         Q, K, V = (t.permute(0, 2, 1, 3).double() for t in (q, k, v))
