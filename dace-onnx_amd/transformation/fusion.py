@@ -199,7 +199,11 @@ def _fold_into_contractions(sdfg: SDFG, state: SDFGState) -> int:
                         folded += 1
                         changed = True
                         break
-            # ---- activation
+            # ---- activation (it runs before the residual in the epilogue: a Gemm whose C is a full [M, N]
+            # addend, which the expansion passes as the residual, cannot take one)
+            if _is_op(node, "Gemm") and _in_edge(state, node, "C") is not None:
+                c_shape = tuple(sdfg.arrays[_in_edge(state, node, "C").src.data].shape)
+                has_res = has_res or not (len(c_shape) == 1 or (len(c_shape) == 2 and c_shape[0] == 1))
             if _is_op(nxt, "Relu", "Gelu") and not has_res and act is None:
                 is_gelu = _is_op(nxt, "Gelu")
                 if (not is_gelu or ((nxt.approximate or "none") == "none" and not _is_op(node, "Conv"))):

@@ -329,3 +329,22 @@ def test_bert_layer_other_sequence_lengths(seq):
     got = model(x)
     assert model.compile_and_init().num_launches == 7
     assert rel_err(O.bert_layer(x, w, heads=4), got) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("c_shape", [(12, ), (6, 12)])
+@pytest.mark.parametrize("act", ["Relu", "Gelu"])
+def test_gemm_addend_then_activation(c_shape, act):
+    # act(A B + C): a row bias folds with the activation into one launch; a full [M, N] addend must be added
+    # before the activation, so the activation stays its own launch (the epilogue adds a residual last)
+    H, T = proto.helper, proto.TensorProto
+    rng = np.random.default_rng(len(c_shape))
+    a, b, c = (rng.normal(size=s).astype(np.float32) for s in ((6, 8), (8, 12), c_shape))
+    nodes = [H.make_node("Gemm", ["a", "b", "c"], ["g"]), H.make_node(act, ["g"], ["y"])]
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("a", T.FLOAT, [6, 8]), H.make_tensor_value_info("b", T.FLOAT, [8, 12]),
+                                  H.make_tensor_value_info("c", T.FLOAT, list(c_shape))],
+                     [H.make_tensor_value_info("y", T.FLOAT, [6, 12])])
+    model = donnx.ONNXModel(f"gemm_{act}_{len(c_shape)}", H.make_model(g, opset_imports=[H.make_opsetid("", 12)]))
+    got = model(a, b, c)
+    pre = O.gemm(a, b, c)
+    assert rel_err(O.relu(pre) if act == "Relu" else O.gelu(pre), got) < FP32_REL_TOL
+    assert model.compile_and_init().num_launches == (1 if len(c_shape) == 1 else 2)

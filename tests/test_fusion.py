@@ -193,3 +193,18 @@ def test_scalar_scale_on_an_operand_becomes_alpha():
         assert alpha in calls[0][1]
     # a constant numerator is not a scale of the operand: c / q stays an elementwise launch
     assert [f for f, _ in _launches(model("Div", True))] == ["mi355x_eltwise_f32", "mi355x_gemm_f32"]
+
+
+def test_gemm_with_a_full_addend_does_not_take_an_activation():
+    # the epilogue order is bias, activation, residual; Gemm's C of shape [M, N] travels as the residual, so
+    # Relu(A B + C) must stay two launches, while a row bias C of shape [N] folds
+    T = proto.TensorProto
+    def model(c_shape):
+        nodes = [H.make_node("Gemm", ["a", "b", "c"], ["g"]), H.make_node("Relu", ["g"], ["y"])]
+        g = H.make_graph(nodes, "g", [H.make_tensor_value_info("a", T.FLOAT, [6, 8]), H.make_tensor_value_info("b", T.FLOAT, [8, 12]),
+                                      H.make_tensor_value_info("c", T.FLOAT, c_shape)],
+                         [H.make_tensor_value_info("y", T.FLOAT, [6, 12])])
+        return donnx.ONNXModel("gemm_relu_" + str(len(c_shape)), H.make_model(g, opset_imports=[H.make_opsetid("", 12)]))
+    assert [f for f, _ in _launches(model([12]))] == ["mi355x_gemm_f32"]
+    assert [f for f, _ in _launches(model([1, 12]))] == ["mi355x_gemm_f32"]
+    assert [f for f, _ in _launches(model([6, 12]))] == ["mi355x_gemm_f32", "mi355x_eltwise_f32"]
