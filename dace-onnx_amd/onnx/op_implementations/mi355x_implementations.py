@@ -665,3 +665,18 @@ def _alias_impl(op_name, in_conn, out_conn):
 MI355XReshape = _alias_impl("Reshape", "data", "reshaped")
 MI355XFlatten = _alias_impl("Flatten", "input", "output")
 MI355XIdentity = _alias_impl("Identity", "input", "output")
+
+
+@op_implementation(op="Pad", name=IMPLEMENTATION_NAME)
+class MI355XPad(ONNXForward):
+    """No kernel of its own: a constant zero Pad of the spatial axes is folded into the Conv that reads
+    it before expansion (``transformation/fusion.py``, the reference's ``PadConvFusion``). A Pad that is
+    still in the graph at expansion time is refused, which the reference would hand to ONNX Runtime."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        return False
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        raise NotImplementedError("Pad is only supported folded into a Conv")

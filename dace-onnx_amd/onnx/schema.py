@@ -132,6 +132,12 @@ SCHEMAS: typing.List[ONNXSchema] = [
     _unary("Transpose", 1, "data", "transposed", types=_ANY, attributes=[ONNXAttribute("perm", _A.Ints)]),
     _unary("Flatten", 11, "input", "output", types=_ANY, attributes=[ONNXAttribute("axis", _A.Int, 1)]),
     _unary("Identity", 1, "input", "output", types=_ANY),
+    # Pad only ever runs folded into the Conv that reads it (transformation/fusion.py, the reference's PadConvFusion)
+    ONNXSchema("Pad", 11,
+               [ONNXParameter("data", "T"), ONNXParameter("pads", "tensor(int64)"), ONNXParameter("constant_value", "T", _O)],
+               [ONNXParameter("output", "T")], [ONNXAttribute("mode", _A.String, "constant")],
+               [ONNXTypeConstraint("T", _NUMERIC), ONNXTypeConstraint("tensor(int64)", [dace.int64])],
+               "Pad `data` by `pads` = [begin_0, ..., begin_n, end_0, ..., end_n]."),
     # Not an ONNX operator: the node the fusion pass puts in place of MatMul -> scale -> Softmax -> MatMul.
     ONNXSchema("FusedAttention", 1,
                [ONNXParameter("Q", "T"), ONNXParameter("K", "T"), ONNXParameter("V", "T")], [ONNXParameter("O", "T")],

@@ -87,6 +87,14 @@ def _infer_node(node, shapes, types, constants):
         if int(np.prod(out)) != total:
             raise ShapeInferenceError(f"Reshape '{node.name}': cannot reshape {ins[0]} to {target}")
         return [(tuple(out), tys[0])]
+    if op == "Pad":
+        if node.input[1] not in constants:
+            raise ShapeInferenceError(f"Pad '{node.name}': the pads input must be a constant initializer")
+        pads = [int(v) for v in constants[node.input[1]].ravel()]
+        rank = len(ins[0])
+        if len(pads) != 2 * rank:
+            raise ShapeInferenceError(f"Pad '{node.name}': {len(pads)} pads for a rank-{rank} input")
+        return [(tuple(ins[0][i] + pads[i] + pads[i + rank] for i in range(rank)), tys[0])]
     if op == "Flatten":
         axis = a.get("axis", 1) % (len(ins[0]) + 1) if a.get("axis", 1) < 0 else a.get("axis", 1)
         return [((int(np.prod(ins[0][:axis])) if axis else 1, int(np.prod(ins[0][axis:]))), tys[0])]

@@ -24,6 +24,7 @@ MatMul -> Transpose -> Reshape               MatMul writes the final array throu
 ReduceMean, Sub, Pow(2), ReduceMean,         LayerNormalization (what exporters below
 Add(eps), Sqrt, Div, Mul(gamma), Add(beta)   opset 17 write for ``nn.LayerNorm``)
 Div(sqrt 2), Erf, Add(1), Mul(x), Mul(0.5)   Gelu (exact erf form, any operand order)
+Pad(constant 0, spatial) -> Conv             the Conv's ``pads`` grow (``PadConvFusion``)
 MatMul(alpha) -> Softmax(last) -> MatMul     FusedAttention when the kernel supports the
                                              shape (head size 64)
 MatMuls of one A with constant weights       one MatMul with the weights (and biases)
@@ -149,6 +150,43 @@ def _replace_output(sdfg, state, node, out_conn, folded_node, folded_out_conn):
     state.remove_node(folded_node)
     state.remove_node(mid_access)
     del sdfg.arrays[mid_access.data]
+
+
+def _fuse_pad_conv(sdfg: SDFG, state: SDFGState) -> int:
+    """A constant zero ``Pad`` of the spatial axes whose only reader is a ``Conv`` becomes part of the
+    convolution's ``pads`` (the reference's ``PadConvFusion``, ``daceml/transformation/pad_conv_fusion.py``:
+    constant mode, value 0, 4-D, eight constant pads, nothing padded along batch or channels)."""
+    fused = 0
+    for pad in list(state.nodes()):
+        if not _is_op(pad, "Pad") or (pad.mode or "constant") != "constant":
+            continue
+        out_e, data_e, pads_e = _out_edge(state, pad, "output"), _in_edge(state, pad, "data"), _in_edge(state, pad, "pads")
+        if out_e is None or data_e is None or pads_e is None or not isinstance(out_e.dst, AccessNode):
+            continue
+        use = _single_consumer(sdfg, state, out_e.dst)
+        if use is None or not _is_op(use.dst, "Conv") or use.dst_conn != "X" or len(sdfg.arrays[out_e.dst.data].shape) != 4:
+            continue
+        conv = use.dst
+        pads = _constant_value(sdfg, pads_e.src.data)
+        value_e = _in_edge(state, pad, "constant_value")
+        value = _constant_value(sdfg, value_e.src.data) if value_e is not None else np.zeros(1)
+        if pads is None or pads.size != 8 or value is None or value.size != 1 or float(value.reshape(-1)[0]) != 0.0:
+            continue
+        pads = [int(v) for v in pads.reshape(-1)]
+        if any(pads[i] != 0 for i in (0, 1, 4, 5)) or min(pads) < 0:
+            continue
+        if (conv.auto_pad or "NOTSET") != "NOTSET":
+            continue
+        old = list(conv.pads) if conv.pads is not None else [0, 0, 0, 0]
+        conv.pads = [old[0] + pads[2], old[1] + pads[3], old[2] + pads[6], old[3] + pads[7]]
+        mid = out_e.dst
+        state.remove_edge(use)
+        state.add_edge(data_e.src, None, conv, "X", sdfg.make_array_memlet(data_e.src.data))
+        state.remove_node(pad)
+        state.remove_node(mid)
+        del sdfg.arrays[mid.data]
+        fused += 1
+    return fused
 
 
 def _fold_into_contractions(sdfg: SDFG, state: SDFGState) -> int:
@@ -926,6 +964,7 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
     """Apply every fusion pattern to every state; returns the number of folds."""
     total = 0
     for state in sdfg.nodes():
+        total += _fuse_pad_conv(sdfg, state)
         total += _fuse_decomposed_layernorm(sdfg, state)
         total += _fuse_decomposed_gelu(sdfg, state)
         total += _fold_into_contractions(sdfg, state)

@@ -348,3 +348,17 @@ def test_gemm_addend_then_activation(c_shape, act):
     pre = O.gemm(a, b, c)
     assert rel_err(O.relu(pre) if act == "Relu" else O.gelu(pre), got) < FP32_REL_TOL
     assert model.compile_and_init().num_launches == (1 if len(c_shape) == 1 else 2)
+
+
+def test_pad_then_conv_matches_padding_by_hand():
+    # Pad(constant 0, spatial) -> Conv(pads) -> Relu as one convolution launch, against the oracle's convolution
+    # of the explicitly padded input
+    from test_fusion import _pad_conv_model
+    m = _pad_conv_model([0, 0, 1, 2, 0, 0, 3, 0], conv_pads=[1, 0, 0, 2])
+    x = np.random.default_rng(6).normal(size=(2, 3, 8, 8)).astype(np.float32)
+    w = [t for t in m.graph.initializer if t.name == "w"][0].array.reshape(4, 3, 3, 3)
+    model = donnx.ONNXModel("pad_conv_values", m)
+    got = model(x)
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 3), (2, 0)))
+    assert rel_err(O.conv2d(xp, w, None, pads=(1, 0, 0, 2)), got) < FP32_REL_TOL
+    assert model.compile_and_init().num_launches == 1

@@ -208,3 +208,38 @@ def test_gemm_with_a_full_addend_does_not_take_an_activation():
     assert [f for f, _ in _launches(model([12]))] == ["mi355x_gemm_f32"]
     assert [f for f, _ in _launches(model([1, 12]))] == ["mi355x_gemm_f32"]
     assert [f for f, _ in _launches(model([6, 12]))] == ["mi355x_gemm_f32", "mi355x_eltwise_f32"]
+
+
+def _pad_conv_model(pads, value=0.0, mode="constant", conv_pads=None, second_reader=False):
+    T = proto.TensorProto
+    rng = np.random.default_rng(5)
+    inits = [proto.numpy_helper.from_array(np.array(pads, np.int64), name="pads"),
+             proto.numpy_helper.from_array(np.array(value, np.float32), name="zero"),
+             proto.numpy_helper.from_array(rng.normal(size=(4, 3, 3, 3)).astype(np.float32), name="w")]
+    out_hw = [8 + pads[2] + pads[6] + (conv_pads[0] + conv_pads[2] if conv_pads else 0) - 2,
+              8 + pads[3] + pads[7] + (conv_pads[1] + conv_pads[3] if conv_pads else 0) - 2]
+    attrs = {"pads": conv_pads} if conv_pads else {}
+    nodes = [H.make_node("Pad", ["x", "pads", "zero"], ["xp"], mode=mode), H.make_node("Conv", ["xp", "w"], ["y"], **attrs)]
+    outs = [H.make_tensor_value_info("y", T.FLOAT, [2, 4] + out_hw)]
+    if second_reader:
+        nodes.append(H.make_node("Relu", ["xp"], ["r"]))
+        outs.append(H.make_tensor_value_info("r", T.FLOAT, None))
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("x", T.FLOAT, [2, 3, 8, 8])], outs, initializer=inits)
+    return H.make_model(g, opset_imports=[H.make_opsetid("", 12)])
+
+
+def test_pad_conv_fusion():
+    # the reference's PadConvFusion: a constant zero pad of H and W folds into the convolution's pads
+    calls = _launches(donnx.ONNXModel("pad_conv", _pad_conv_model([0, 0, 1, 2, 0, 0, 3, 0])))
+    assert [f for f, _ in calls] == ["mi355x_conv2d_f32"]
+    assert [1, 2, 3, 0] in calls[0][1]                       # pads {top, left, bottom, right}
+    calls = _launches(donnx.ONNXModel("pad_conv2", _pad_conv_model([0, 0, 1, 1, 0, 0, 1, 1], conv_pads=[1, 0, 0, 2])))
+    assert [2, 1, 1, 3] in calls[0][1]                       # added to the pads the Conv already had
+    # not foldable: a non-zero value, another mode, padding along channels, a second reader of the padded tensor;
+    # a Pad that stays has no kernel here and is refused when it is expanded
+    from dace_onnx_amd.onnx.nodes.onnx_op import ExpansionRefused
+    for kwargs in (dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], value=1.0), dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], mode="reflect"),
+                   dict(pads=[0, 1, 1, 1, 0, 0, 1, 1]), dict(pads=[0, 0, 1, 1, 0, 0, 1, 1], second_reader=True)):
+        model = donnx.ONNXModel("pad_kept", _pad_conv_model(**kwargs))
+        with pytest.raises(ExpansionRefused, match="Pad"):
+            model.expand()
