@@ -20,7 +20,9 @@ LIBRARY_PATH = os.path.join(_HERE, LIBRARY_NAME)
 OK = 0
 EPI_NONE, EPI_BIAS, EPI_RELU, EPI_GELU, EPI_RESIDUAL = 0, 1, 2, 4, 8
 OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_POW = 0, 1, 2, 3, 4
-OP_RELU, OP_GELU, OP_ERF, OP_SQRT = 16, 17, 18, 19
+OP_RELU, OP_GELU, OP_ERF, OP_SQRT, OP_COPY = 16, 17, 18, 19, 20
+PROGRAM_REG, PROGRAM_TENSOR, PROGRAM_VECTOR, PROGRAM_IMMEDIATE = 0, 1, 2, 3
+PROGRAM_MAX_INSTR, PROGRAM_MAX_TENSORS, PROGRAM_MAX_VECTORS, PROGRAM_MAX_IMM = 16, 4, 4, 8
 
 _c_i64_p = ctypes.POINTER(ctypes.c_int64)
 _vp = ctypes.c_void_p
@@ -47,6 +49,9 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
     "mi355x_reduce_mean_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_eltwise_f32": (_int, [_int, _vp, _vp, _vp, _int, _c_i64_p, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_permute_b32": (_int, [_vp, _vp, _int, _c_i64_p, _c_i64_p, _vp]),
+    "mi355x_eltwise_program_f32": (_int, [ctypes.POINTER(ctypes.c_void_p), _int, ctypes.POINTER(ctypes.c_void_p), _int, _vp,
+                                          _i64, _i64, ctypes.POINTER(ctypes.c_uint32), _int,
+                                          ctypes.POINTER(ctypes.c_float), _int, _vp]),
 }
 
 
@@ -86,6 +91,18 @@ def check(status: int, what: str) -> None:
 
 def i64_array(values: typing.Sequence[int]):
     return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+
+
+def u32_array(values: typing.Sequence[int]):
+    return (ctypes.c_uint32 * max(len(values), 1))(*[int(v) for v in values])
+
+
+def f32_array(values: typing.Sequence[float]):
+    return (ctypes.c_float * max(len(values), 1))(*[float(v) for v in values])
+
+
+def pointer_array(addresses: typing.Sequence[int]):
+    return (ctypes.c_void_p * max(len(addresses), 1))(*[int(a) for a in addresses])
 
 
 def current_stream() -> int:

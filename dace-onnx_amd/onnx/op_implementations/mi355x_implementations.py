@@ -32,7 +32,7 @@ import numpy as np
 
 from ... import sdfg as dace
 from ... import _lib
-from ...sdfg import SDFG, SDFGState, Ptr, Stream, I64Array, AliasNode
+from ...sdfg import SDFG, SDFGState, Ptr, Stream, I64Array, U32Array, F32Array, PtrArray, AliasNode
 from ...util.utils import in_desc_with_name, out_desc_with_name, prod
 from ..forward_implementation_abc import ONNXForward
 from .utils import op_implementation, kernel_call_for_node
@@ -680,3 +680,44 @@ class MI355XPad(ONNXForward):
     @staticmethod
     def forward(node, state: SDFGState, sdfg: SDFG):
         raise NotImplementedError("Pad is only supported folded into a Conv")
+
+
+@op_implementation(op="FusedElementwise", name=IMPLEMENTATION_NAME)
+class MI355XFusedElementwise(ONNXForward):
+    """A group of elementwise nodes merged by the fusion pass: one launch of the program kernel. Inputs
+    ``X__i`` are tensors of the output's shape (``kinds[i] == 1``) or vectors along the last axis (2)."""
+
+    @staticmethod
+    def _inputs(node, state, sdfg):
+        conns = sorted((c for c in node.in_connectors if c.startswith("X__")), key=lambda c: int(c[3:]))
+        kinds = list(node.kinds or [])
+        return conns, kinds
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        conns, kinds = MI355XFusedElementwise._inputs(node, state, sdfg)
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        if len(conns) != len(kinds) or not conns or not _is_f32(Y) or not Y.is_contiguous() or not node.program:
+            return False
+        for c, k in zip(conns, kinds):
+            d = in_desc_with_name(node, state, sdfg, c)
+            if not _is_f32(d) or not d.is_contiguous():
+                return False
+            if k == _lib.PROGRAM_TENSOR and tuple(d.shape) != tuple(Y.shape):
+                return False
+            if k == _lib.PROGRAM_VECTOR and (not Y.shape or d.total_size != Y.shape[-1]):
+                return False
+        return kinds.count(_lib.PROGRAM_TENSOR) <= _lib.PROGRAM_MAX_TENSORS and \
+            kinds.count(_lib.PROGRAM_VECTOR) <= _lib.PROGRAM_MAX_VECTORS and \
+            len(node.program) <= _lib.PROGRAM_MAX_INSTR and len(node.immediates or []) <= _lib.PROGRAM_MAX_IMM
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        conns, kinds = MI355XFusedElementwise._inputs(node, state, sdfg)
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        tensors = [c for c, k in zip(conns, kinds) if k == _lib.PROGRAM_TENSOR]
+        vectors = [c for c, k in zip(conns, kinds) if k == _lib.PROGRAM_VECTOR]
+        imms = list(node.immediates or [])
+        return kernel_call_for_node(node, state, "mi355x_eltwise_program_f32", [
+            PtrArray(tensors), len(tensors), PtrArray(vectors), len(vectors), Ptr("Y"), int(Y.total_size),
+            int(Y.shape[-1]) if Y.shape else 1, U32Array(node.program), len(node.program), F32Array(imms), len(imms), Stream()])

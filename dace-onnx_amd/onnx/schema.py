@@ -143,6 +143,11 @@ SCHEMAS: typing.List[ONNXSchema] = [
                [ONNXParameter("Q", "T"), ONNXParameter("K", "T"), ONNXParameter("V", "T")], [ONNXParameter("O", "T")],
                [ONNXAttribute("scale", _A.Float, 1.0)], [ONNXTypeConstraint("T", [dace.float32])],
                "softmax(scale * Q K^T) V per batch entry; Q, O are [..., Sq, D], K, V are [..., Sk, D]."),
+    # Not an ONNX operator: a group of elementwise nodes merged by the fusion pass into one launch.
+    ONNXSchema("FusedElementwise", 1, [ONNXParameter("X", "T", ONNXParameterType.Variadic)], [ONNXParameter("Y", "T")],
+               [ONNXAttribute("program", _A.Ints), ONNXAttribute("immediates", _A.Floats), ONNXAttribute("kinds", _A.Ints)],
+               [ONNXTypeConstraint("T", [dace.float32])],
+               "Y = program(X__0, X__1, ...): instructions, immediates and operand kinds as in mi355x_eltwise_program_f32."),
     ONNXSchema("Pow", 12, [ONNXParameter("X", "T"), ONNXParameter("Y", "T1")], [ONNXParameter("Z", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64]), ONNXTypeConstraint("T1", _NUMERIC)]),
     ONNXSchema("ReduceMean", 11, [ONNXParameter("data", "T")], [ONNXParameter("reduced", "T")],

@@ -262,6 +262,36 @@ class I64Array:
         return f"I64Array({self.values})"
 
 
+class U32Array:
+    """Kernel argument: a small constant ``const uint32_t[]`` (an elementwise program)."""
+
+    def __init__(self, values):
+        self.values = [int(v) & 0xFFFFFFFF for v in values]
+
+    def __repr__(self):
+        return f"U32Array({[hex(v) for v in self.values]})"
+
+
+class F32Array:
+    """Kernel argument: a small constant ``const float[]`` (immediates of an elementwise program)."""
+
+    def __init__(self, values):
+        self.values = [float(v) for v in values]
+
+    def __repr__(self):
+        return f"F32Array({self.values})"
+
+
+class PtrArray:
+    """Kernel argument: ``const float* const[]`` built from the arrays attached to several connectors."""
+
+    def __init__(self, connectors):
+        self.connectors = list(connectors)
+
+    def __repr__(self):
+        return f"PtrArray({self.connectors})"
+
+
 class KernelCall(Node):
     """One call into ``libmi355x_onnx.so``; what a ``"mi355x"`` expansion returns.
 
@@ -290,6 +320,15 @@ class KernelCall(Node):
                 call_args.append("__dace_current_stream")
             elif isinstance(a, I64Array):
                 lines.append(f"const int64_t __arg{i}[] = {{{', '.join(str(v) for v in a.values)}}};")
+                call_args.append(f"__arg{i}")
+            elif isinstance(a, U32Array):
+                lines.append(f"const uint32_t __arg{i}[] = {{{', '.join(hex(v) + 'u' for v in a.values) or '0u'}}};")
+                call_args.append(f"__arg{i}")
+            elif isinstance(a, F32Array):
+                lines.append(f"const float __arg{i}[] = {{{', '.join(repr(v) + 'f' for v in a.values) or '0.0f'}}};")
+                call_args.append(f"__arg{i}")
+            elif isinstance(a, PtrArray):
+                lines.append(f"const float* const __arg{i}[] = {{{', '.join('_' + c for c in a.connectors) or 'nullptr'}}};")
                 call_args.append(f"__arg{i}")
             elif a is None:
                 call_args.append("nullptr")
@@ -647,6 +686,13 @@ class CompiledSDFG:
                     args.append(None)
                 elif isinstance(a, I64Array):
                     arr = _lib.i64_array(a.values)
+                    keep.append(arr)
+                    args.append(arr)
+                elif isinstance(a, (U32Array, F32Array, PtrArray)):
+                    if isinstance(a, PtrArray):
+                        arr = _lib.pointer_array([env[conn_to_key[c]].data_ptr() for c in a.connectors])
+                    else:
+                        arr = (_lib.u32_array if isinstance(a, U32Array) else _lib.f32_array)(a.values)
                     keep.append(arr)
                     args.append(arr)
                 else:

@@ -45,6 +45,8 @@ import typing
 
 import numpy as np
 
+from .. import _lib
+
 from ..sdfg import SDFG, SDFGState, AccessNode, Array, _contiguous_strides
 
 log = logging.getLogger(__name__)
@@ -934,6 +936,141 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
     return fused
 
 
+_EW_BINARY = {"Add": _lib.OP_ADD, "Sub": _lib.OP_SUB, "Mul": _lib.OP_MUL, "Div": _lib.OP_DIV, "Pow": _lib.OP_POW}
+_EW_UNARY = {"Relu": _lib.OP_RELU, "Gelu": _lib.OP_GELU, "Erf": _lib.OP_ERF, "Sqrt": _lib.OP_SQRT, "Identity": _lib.OP_COPY}
+
+
+class _ProgramTooLarge(Exception):
+    pass
+
+
+def _fuse_elementwise(sdfg: SDFG, state: SDFGState) -> int:
+    """Groups of elementwise nodes (Add, Sub, Mul, Div, Pow, Relu, Gelu, Erf, Sqrt, Identity) whose
+    intermediate results have one reader become one ``FusedElementwise`` node: a short program for
+    ``mi355x_eltwise_program_f32`` in which every tensor operand is read once and only the final result is
+    written -- what the reference leaves to DaCe's map / tasklet fusion after expansion
+    (``daceml/transformation/tasklet_fusion.py``). A group is grown backwards from its last node; an operand
+    is another member's result, a tensor of the result's shape, a vector along the last axis, or a scalar
+    constant. Runs last, on whatever the GEMM / Conv epilogue folds and the pattern rewrites left over."""
+    from ..onnx.nodes.onnx_op import get_onnx_node
+
+    def fusable(n):
+        if _is_op(n, *_EW_BINARY):
+            return True
+        if _is_op(n, "Gelu"):
+            return (n.approximate or "none") == "none"
+        return _is_op(n, *_EW_UNARY)
+
+    def io_edges(n):
+        ins = [_in_edge(state, n, prm.name) for prm in n.schema.inputs]
+        return ins, _out_edge(state, n, n.schema.outputs[0].name)
+
+    def f32_contiguous(desc):
+        return desc.dtype.name == "float32" and desc.is_contiguous()
+
+    done = set()
+    fused = 0
+    for final in reversed(list(state.topological_nodes())):
+        if final in done or not fusable(final):
+            continue
+        ins, out_e = io_edges(final)
+        if out_e is None or not isinstance(out_e.dst, AccessNode) or any(e is None for e in ins):
+            continue
+        shape = tuple(sdfg.arrays[out_e.dst.data].shape)
+        if not shape or not f32_contiguous(sdfg.arrays[out_e.dst.data]):
+            continue
+        members, tensors, vectors, imms, program = [], [], [], [], []
+        free_regs = list(range(8))
+
+        def operand(edge):
+            """Encoded operand for the value on ``edge``; absorbs its producer when it can join the group."""
+            acc = edge.src
+            desc = sdfg.arrays[acc.data]
+            const = _constant_value(sdfg, acc.data) if not state.in_edges(acc) else None
+            if const is not None and const.size == 1 and const.dtype == np.float32:
+                v = float(const.reshape(-1)[0])
+                if v not in imms:
+                    imms.append(v)
+                return (_lib.PROGRAM_IMMEDIATE << 6) | imms.index(v), None
+            prod = _producer(state, acc)
+            if prod is not None and fusable(prod.src) and prod.src not in done and tuple(desc.shape) == shape \
+                    and f32_contiguous(desc) and _single_consumer(sdfg, state, acc) is not None:
+                p_ins, _ = io_edges(prod.src)
+                if all(e is not None for e in p_ins):
+                    # tentative: if the producer (or something it needs) does not fit, it stays outside and
+                    # its result is read as a tensor
+                    snapshot = (len(members), len(program), list(free_regs), len(tensors), len(vectors), len(imms))
+                    try:
+                        reg = emit(prod.src, p_ins)
+                        return (_lib.PROGRAM_REG << 6) | reg, reg
+                    except _ProgramTooLarge:
+                        del members[snapshot[0]:], program[snapshot[1]:], tensors[snapshot[3]:], vectors[snapshot[4]:]
+                        del imms[snapshot[5]:]
+                        free_regs[:] = snapshot[2]
+            if not f32_contiguous(desc):
+                raise _ProgramTooLarge()
+            if tuple(desc.shape) == shape:
+                if acc.data not in tensors:
+                    tensors.append(acc.data)
+                return (_lib.PROGRAM_TENSOR << 6) | tensors.index(acc.data), None
+            if desc.total_size == shape[-1] and desc.shape and desc.shape[-1] == shape[-1]:
+                if acc.data not in vectors:
+                    vectors.append(acc.data)
+                return (_lib.PROGRAM_VECTOR << 6) | vectors.index(acc.data), None
+            raise _ProgramTooLarge()     # a broadcast this kernel does not do
+
+        def emit(n, in_edges):
+            encoded = [operand(e) for e in in_edges]
+            for _, reg in encoded:
+                if reg is not None:
+                    free_regs.append(reg)       # an intermediate has exactly one reader: this instruction
+            if not free_regs:
+                raise _ProgramTooLarge()
+            dst = min(free_regs)
+            free_regs.remove(dst)
+            a = encoded[0][0]
+            b = encoded[1][0] if len(encoded) > 1 else 0
+            if _is_op(n, "Pow") and (b >> 6) == _lib.PROGRAM_IMMEDIATE and imms[b & 63] == 2.0:
+                op, b = _lib.OP_MUL, a
+            else:
+                op = _EW_BINARY.get(n.schema.name, _EW_UNARY.get(n.schema.name))
+            program.append(op | (dst << 8) | (a << 16) | (b << 24))
+            members.append(n)
+            if len(program) > _lib.PROGRAM_MAX_INSTR or len(tensors) > _lib.PROGRAM_MAX_TENSORS or \
+                    len(vectors) > _lib.PROGRAM_MAX_VECTORS or len(imms) > _lib.PROGRAM_MAX_IMM:
+                raise _ProgramTooLarge()
+            return dst
+
+        try:
+            emit(final, ins)
+        except _ProgramTooLarge:
+            continue
+        if len(members) < 2 or not (tensors or vectors):
+            continue
+        # ---- rewrite
+        node = get_onnx_node("FusedElementwise")(final.label + "_fused", program=list(program), immediates=list(imms),
+                                                 kinds=[_lib.PROGRAM_TENSOR] * len(tensors) + [_lib.PROGRAM_VECTOR] * len(vectors))
+        state.add_node(node)
+        accesses = {}
+        for m in members:
+            for e in state.in_edges(m):
+                accesses.setdefault(e.src.data, e.src)
+        for i, name in enumerate(tensors + vectors):
+            node.add_in_connector(f"X__{i}")
+            state.add_edge(accesses[name], None, node, f"X__{i}", sdfg.make_array_memlet(name))
+        node.add_out_connector("Y")
+        state.add_edge(node, "Y", out_e.dst, None, sdfg.make_array_memlet(out_e.dst.data))
+        intermediates = [_out_edge(state, m, m.schema.outputs[0].name).dst for m in members if m is not final]
+        for m in members:
+            state.remove_node(m)
+            done.add(m)
+        for acc in intermediates:
+            state.remove_node(acc)
+            del sdfg.arrays[acc.data]
+        fused += len(members) - 1
+    return fused
+
+
 def _remove_dead_nodes(sdfg: SDFG, state: SDFGState) -> int:
     """Drop nodes whose outputs nobody reads (left behind by the view folds)."""
     removed = 0
@@ -974,6 +1111,8 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
         total += _fuse_attention(sdfg, state)
         total += _fuse_shared_input_matmuls(sdfg, state)
         total += _pretranspose_weights(sdfg, state)
+        _remove_dead_nodes(sdfg, state)
+        total += _fuse_elementwise(sdfg, state)
         _remove_dead_nodes(sdfg, state)
     if total:
         log.info("fused %d patterns in SDFG %s", total, sdfg.name)

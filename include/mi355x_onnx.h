@@ -187,6 +187,32 @@ int mi355x_eltwise_f32(int op, const float* A, const float* B, float* C,
                        const int64_t* a_strides, const int64_t* b_strides,
                        void* stream);
 
+/* A group of elementwise nodes as one launch, fp32: every tensor operand is read once, the result
+ * written once, intermediates stay in registers. In the reference each of these nodes is its own map with
+ * a materialised result (pure_implementations.py:41-127, 462-474) and merging them is left to DaCe's map /
+ * tasklet fusion (daceml/transformation/tasklet_fusion.py); here the fusion pass emits a short program.
+ *   tensors[n_tensors]  inputs of the result's shape, C-contiguous (n elements each)
+ *   vectors[n_vectors]  inputs of last_dim elements, broadcast along every other axis
+ *   immediates          scalar constants (host memory, copied into the launch)
+ *   program[n_instr]    host memory; one 32-bit word per instruction:
+ *                         op | dst register << 8 | operand a << 16 | operand b << 24
+ *                       op is one of MI355X_OP_* (unary ops ignore b); registers are 0..7; an operand byte is
+ *                       kind << 6 | index with the kinds below. Y receives the last instruction's result.
+ * Limits are the MI355X_PROGRAM_MAX_* below; a register must be written before it is read. */
+#define MI355X_OP_COPY 20
+#define MI355X_PROGRAM_REG 0
+#define MI355X_PROGRAM_TENSOR 1
+#define MI355X_PROGRAM_VECTOR 2
+#define MI355X_PROGRAM_IMMEDIATE 3
+#define MI355X_PROGRAM_MAX_INSTR 16
+#define MI355X_PROGRAM_MAX_TENSORS 4
+#define MI355X_PROGRAM_MAX_VECTORS 4
+#define MI355X_PROGRAM_MAX_IMM 8
+int mi355x_eltwise_program_f32(const float* const* tensors, int n_tensors,
+                               const float* const* vectors, int n_vectors, float* Y, int64_t n,
+                               int64_t last_dim, const uint32_t* program, int n_instr,
+                               const float* immediates, int n_immediates, void* stream);
+
 /* ONNX Transpose (and any strided gather), 4-byte elements:
  *   Y (C-contiguous, `shape`) [i0..] = X[sum_d i_d * x_strides[d]].
  * Replaces PureTranspose.forward (pure_implementations.py:369-379). ndim <= 8. */

@@ -400,3 +400,46 @@ def test_torch_tensors_stay_on_device():
     donnx.ONNXSoftmax(input=x, output=y, axis=-1)
     torch.cuda.synchronize()
     assert rel_err(O.softmax(x.cpu().numpy()), y.cpu().numpy()) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- elementwise programs
+def _ins(op, dst, a, b=0):
+    return op | (dst << 8) | (a << 16) | (b << 24)
+
+
+def _opnd(kind, idx):
+    return (kind << 6) | idx
+
+
+@pytest.mark.parametrize("shape", [(6, 40, 768), (5, 7, 9), (1, 4), (3, 1)])
+def test_eltwise_program_c_abi(shape):
+    # y = gelu((t0 * 0.5 + v0) / t1) - relu(v1 * t0): tensors, vectors along the last axis, immediates, registers
+    R, TN, VC, IM = _lib.PROGRAM_REG, _lib.PROGRAM_TENSOR, _lib.PROGRAM_VECTOR, _lib.PROGRAM_IMMEDIATE
+    rng = np.random.default_rng(sum(shape))
+    t0 = rng.normal(size=shape).astype(np.float32)
+    t1 = (rng.random(size=shape) + 0.5).astype(np.float32)
+    v0, v1 = rng.normal(size=shape[-1]).astype(np.float32), rng.normal(size=shape[-1]).astype(np.float32)
+    program = [_ins(_lib.OP_MUL, 0, _opnd(TN, 0), _opnd(IM, 0)),
+               _ins(_lib.OP_ADD, 0, _opnd(R, 0), _opnd(VC, 0)),
+               _ins(_lib.OP_DIV, 1, _opnd(R, 0), _opnd(TN, 1)),
+               _ins(_lib.OP_GELU, 1, _opnd(R, 1)),
+               _ins(_lib.OP_MUL, 2, _opnd(VC, 1), _opnd(TN, 0)),
+               _ins(_lib.OP_RELU, 2, _opnd(R, 2)),
+               _ins(_lib.OP_SUB, 0, _opnd(R, 1), _opnd(R, 2))]
+    expected = O.sub(O.gelu(O.div(O.add(O.mul(t0, np.float32(0.5)), v0), t1)), O.relu(O.mul(v1, t0)))
+    dt = [torch.from_numpy(a).cuda() for a in (t0, t1, v0, v1)]
+    y = torch.full(shape, float("nan"), device="cuda")
+    lib = _lib.library()
+    call = lambda prog, n_t=2, n_v=2, n_imm=1: lib.mi355x_eltwise_program_f32(
+        _lib.pointer_array([dt[0].data_ptr(), dt[1].data_ptr()]), n_t, _lib.pointer_array([dt[2].data_ptr(), dt[3].data_ptr()]),
+        n_v, y.data_ptr(), y.numel(), shape[-1], _lib.u32_array(prog), len(prog), _lib.f32_array([0.5]), n_imm,
+        _lib.current_stream())
+    _lib.check(call(program), "mi355x_eltwise_program_f32")
+    assert rel_err(expected, y.cpu().numpy()) < FP32_REL_TOL
+    # malformed programs are refused before anything is launched: a register read before it is written, an input
+    # that does not exist, an unknown opcode
+    assert call([_ins(_lib.OP_ADD, 0, _opnd(R, 3), _opnd(TN, 0))]) == 1
+    assert "does not exist" in lib.mi355x_last_error().decode()
+    assert call([_ins(_lib.OP_ADD, 0, _opnd(TN, 0), _opnd(VC, 1))], n_v=1) == 1
+    assert call([_ins(9, 0, _opnd(TN, 0), _opnd(TN, 0))]) == 1
+    assert call(program * 3) == 1     # 21 instructions

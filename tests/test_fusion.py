@@ -137,12 +137,18 @@ def test_gelu_pattern_variants():
     for label, nodes in variants.items():
         calls = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))
         assert [(f, a[0]) for f, a in calls] == [("mi355x_eltwise_f32", 17)], label
-    # a different constant is not Gelu: the five nodes stay
+    # a different constant is not Gelu: the five nodes are not replaced by the Gelu node (they still run as one
+    # launch, as a program of five instructions)
     bad = dict(consts, r2=1.5)
-    assert len(_launches(donnx.ONNXModel("g", _chain_model(variants["div, (x * t) * 0.5"], bad)))) == 5
-    # erf(x / sqrt 2) with another reader of the intermediate stays too
+    calls = _launches(donnx.ONNXModel("g", _chain_model(variants["div, (x * t) * 0.5"], bad)))
+    assert [f for f, _ in calls] == ["mi355x_eltwise_program_f32"] and calls[0][1][8] == 5
+    # erf(x / sqrt 2) with another reader of the intermediate is not Gelu either: two programs, split at the
+    # value that has two readers
     nodes = variants["div, (x * t) * 0.5"][:-1] + [mk("Mul", ["u", "e"], ["y"])]
-    assert len(_launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))) == 5
+    calls = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))
+    assert sorted((f, a[8]) for f, a in calls) == [("mi355x_eltwise_program_f32", 2), ("mi355x_eltwise_program_f32", 3)]
+    unfused = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts), fuse=False))
+    assert len(unfused) == 5
 
 
 def test_layernorm_pattern_needs_the_exact_chain():
@@ -157,8 +163,15 @@ def test_layernorm_pattern_needs_the_exact_chain():
 
     calls = _launches(donnx.ONNXModel("ln", _chain_model(chain(), consts)))
     assert [f for f, _ in calls] == ["mi355x_layernorm_f32"] and calls[0][1][6] == pytest.approx(1e-5)
-    assert len(_launches(donnx.ONNXModel("ln3", _chain_model(chain(exponent="three"), consts)))) == 9
-    assert len(_launches(donnx.ONNXModel("ln0", _chain_model(chain(axes=(0, )), dict(consts, g=np.ones(8)))))) == 9
+    # not the LayerNorm chain (cube instead of square; statistics over axis 0): no LayerNormalization node. What
+    # can run as an elementwise program does: Add(eps)+Sqrt, and the tail Mul(gamma)+Add(beta) -- with the Div in
+    # front of it when its divisor is a vector along the last axis (axis-0 statistics) rather than one value
+    # per row, a broadcast the program kernel does not do
+    cube = [f for f, _ in _launches(donnx.ONNXModel("ln3", _chain_model(chain(exponent="three"), consts)))]
+    assert "mi355x_layernorm_f32" not in cube and len(cube) == 7 and cube.count("mi355x_eltwise_program_f32") == 2
+    axis0 = _launches(donnx.ONNXModel("ln0", _chain_model(chain(axes=(0, )), dict(consts, g=np.ones(8)))))
+    assert "mi355x_layernorm_f32" not in [f for f, _ in axis0] and len(axis0) == 6
+    assert sorted(a[8] for f, a in axis0 if f == "mi355x_eltwise_program_f32") == [2, 3]
 
 
 def test_rebase_and_reshape_strides():
