@@ -112,20 +112,23 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p) {
     }
 
     // ---- softmax over the 128 keys of each query row ------------------------------------------------
+    // exp(scale s - max) as 2^(c s - max'), c = scale log2(e): one multiply per score and the bare v_exp_f32
+    // (the library expf costs half a dozen more instructions per value; 32 values per lane)
+    const float c = p.scale * 1.44269504088896340736f;
     float m = -INFINITY;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        acc[j] *= p.scale;
+        acc[j] *= c;
         m = fmaxf(m, fmaxf(fmaxf(acc[j].x, acc[j].y), fmaxf(acc[j].z, acc[j].w)));
     }
     m = quad_lanes_max(m);
     float sum = 0.f;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        acc[j].x = expf(acc[j].x - m);
-        acc[j].y = expf(acc[j].y - m);
-        acc[j].z = expf(acc[j].z - m);
-        acc[j].w = expf(acc[j].w - m);
+        acc[j].x = __builtin_amdgcn_exp2f(acc[j].x - m);
+        acc[j].y = __builtin_amdgcn_exp2f(acc[j].y - m);
+        acc[j].z = __builtin_amdgcn_exp2f(acc[j].z - m);
+        acc[j].w = __builtin_amdgcn_exp2f(acc[j].w - m);
         sum += (acc[j].x + acc[j].y) + (acc[j].z + acc[j].w);
     }
     const float inv = 1.0f / quad_lanes_sum(sum);
@@ -191,6 +194,7 @@ __global__ __launch_bounds__(256) void attention_f32_blocks_kernel(AttnArgs p) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) out[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;   // of query row q0 + li (the same value in its four lanes)
+    const float c = p.scale * 1.44269504088896340736f;   // scores in units of log2: exp(scale s - m) = 2^(c s - m')
 
     for (int64_t key0 = 0; key0 < p.Sk; key0 += SK) {
         f32x4 rk[8], rv[8];
@@ -231,7 +235,7 @@ __global__ __launch_bounds__(256) void attention_f32_blocks_kernel(AttnArgs p) {
         float m_blk = -INFINITY;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            acc[j] *= p.scale;
+            acc[j] *= c;
             if (ragged) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
@@ -240,14 +244,14 @@ __global__ __launch_bounds__(256) void attention_f32_blocks_kernel(AttnArgs p) {
             m_blk = fmaxf(m_blk, fmaxf(fmaxf(acc[j].x, acc[j].y), fmaxf(acc[j].z, acc[j].w)));
         }
         const float m_new = fmaxf(m_run, quad_lanes_max(m_blk));
-        const float alpha = expf(m_run - m_new);    // 0 for the first block
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);    // 0 for the first block
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            acc[j].x = expf(acc[j].x - m_new);
-            acc[j].y = expf(acc[j].y - m_new);
-            acc[j].z = expf(acc[j].z - m_new);
-            acc[j].w = expf(acc[j].w - m_new);
+            acc[j].x = __builtin_amdgcn_exp2f(acc[j].x - m_new);
+            acc[j].y = __builtin_amdgcn_exp2f(acc[j].y - m_new);
+            acc[j].z = __builtin_amdgcn_exp2f(acc[j].z - m_new);
+            acc[j].w = __builtin_amdgcn_exp2f(acc[j].w - m_new);
             sum += (acc[j].x + acc[j].y) + (acc[j].z + acc[j].w);
         }
         l_run = l_run * alpha + quad_lanes_sum(sum);
