@@ -21,6 +21,8 @@ OK = 0
 EPI_NONE, EPI_BIAS, EPI_RELU, EPI_GELU, EPI_RESIDUAL = 0, 1, 2, 4, 8
 OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_POW = 0, 1, 2, 3, 4
 OP_RELU, OP_GELU, OP_ERF, OP_SQRT, OP_COPY = 16, 17, 18, 19, 20
+REDUCE_MEAN, REDUCE_SUM, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
+OP_LOG, OP_TANH, OP_SIGMOID, OP_SOFTPLUS, OP_RECIPROCAL, OP_EXP, OP_NEG, OP_ABS = 21, 22, 23, 24, 25, 26, 27, 28
 PROGRAM_REG, PROGRAM_TENSOR, PROGRAM_VECTOR, PROGRAM_IMMEDIATE = 0, 1, 2, 3
 PROGRAM_MAX_INSTR, PROGRAM_MAX_TENSORS, PROGRAM_MAX_VECTORS, PROGRAM_MAX_IMM = 16, 4, 4, 8
 
@@ -47,6 +49,8 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
                                     _c_i64_p, _c_i64_p, _c_i64_p, _c_i64_p, _f32, _vp]),
     "mi355x_layernorm_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "mi355x_reduce_mean_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_reduce_f32": (_int, [_int, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_log_softmax_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_eltwise_f32": (_int, [_int, _vp, _vp, _vp, _int, _c_i64_p, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_permute_b32": (_int, [_vp, _vp, _int, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_eltwise_program_f32": (_int, [ctypes.POINTER(ctypes.c_void_p), _int, ctypes.POINTER(ctypes.c_void_p), _int, _vp,

@@ -110,6 +110,22 @@ __device__ __forceinline__ float gelu_erf(float v) {
     return 0.5f * v * (1.0f + erf_f32(v * 0.70710678118654752440f));
 }
 
+// The unary maps beyond Relu / Gelu / Erf / Sqrt; `op` is a constant at every call site. Softplus and
+// Sigmoid are written the way the reference writes them (log(1 + exp(x)), 1 / (1 + exp(-x)):
+// pure_implementations.py:696-712), so they also overflow where the reference's do.
+__device__ __forceinline__ float unary_math(int op, float x) {
+    switch (op) {
+        case MI355X_OP_LOG: return logf(x);
+        case MI355X_OP_TANH: return tanhf(x);
+        case MI355X_OP_SIGMOID: return 1.0f / (1.0f + expf(-x));
+        case MI355X_OP_SOFTPLUS: return logf(1.0f + expf(x));
+        case MI355X_OP_RECIPROCAL: return 1.0f / x;
+        case MI355X_OP_EXP: return expf(x);
+        case MI355X_OP_NEG: return -x;
+        default: return fabsf(x);   // MI355X_OP_ABS
+    }
+}
+
 __device__ __forceinline__ float apply_epilogue(float v, int epi, float bias_v) {
     if (epi & MI355X_EPI_BIAS) v += bias_v;
     if (epi & MI355X_EPI_RELU) v = fmaxf(v, 0.0f);

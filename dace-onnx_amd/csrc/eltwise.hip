@@ -1,8 +1,9 @@
-// Elementwise ONNX ops (Add/Sub/Mul/Div, Relu, Gelu, Erf, Sqrt) and the
-// Transpose copy, fp32 / 4-byte elements.
+// Elementwise ONNX ops (Add/Sub/Mul/Div/Pow, Relu, Gelu, Erf, Sqrt, Log, Tanh,
+// Sigmoid, Softplus, Reciprocal, Exp, Neg, Abs) and the Transpose copy, fp32 /
+// 4-byte elements.
 //
 // Each of these is one map in the reference (daceml/onnx/op_implementations/
-// pure_implementations.py:41-56,77-94,112-127,369-379,462-474). They are HBM
+// pure_implementations.py:23-56,77-94,112-127,275-298,369-379,462-474,696-712). They are HBM
 // bound: the kernels below move 16 bytes per lane per access wherever the
 // layout allows and otherwise fall back to an index-decomposing gather.
 //
@@ -32,7 +33,8 @@ __device__ __forceinline__ float apply_op(float a, float b) {
     else if constexpr (OP == MI355X_OP_RELU) return fmaxf(a, 0.0f);
     else if constexpr (OP == MI355X_OP_GELU) return gelu_erf(a);
     else if constexpr (OP == MI355X_OP_ERF) return erff(a);
-    else return sqrtf(a);
+    else if constexpr (OP == MI355X_OP_SQRT) return sqrtf(a);
+    else return unary_math(OP, a);
 }
 template <int OP>
 __device__ __forceinline__ f32x4 apply_op4(f32x4 a, f32x4 b) {
@@ -234,6 +236,14 @@ extern "C" int mi355x_eltwise_f32(int op, const float* A, const float* B, float*
         case MI355X_OP_GELU: return launch_eltwise<MI355X_OP_GELU>(A, B, C, m, st);
         case MI355X_OP_ERF: return launch_eltwise<MI355X_OP_ERF>(A, B, C, m, st);
         case MI355X_OP_SQRT: return launch_eltwise<MI355X_OP_SQRT>(A, B, C, m, st);
+        case MI355X_OP_LOG: return launch_eltwise<MI355X_OP_LOG>(A, B, C, m, st);
+        case MI355X_OP_TANH: return launch_eltwise<MI355X_OP_TANH>(A, B, C, m, st);
+        case MI355X_OP_SIGMOID: return launch_eltwise<MI355X_OP_SIGMOID>(A, B, C, m, st);
+        case MI355X_OP_SOFTPLUS: return launch_eltwise<MI355X_OP_SOFTPLUS>(A, B, C, m, st);
+        case MI355X_OP_RECIPROCAL: return launch_eltwise<MI355X_OP_RECIPROCAL>(A, B, C, m, st);
+        case MI355X_OP_EXP: return launch_eltwise<MI355X_OP_EXP>(A, B, C, m, st);
+        case MI355X_OP_NEG: return launch_eltwise<MI355X_OP_NEG>(A, B, C, m, st);
+        case MI355X_OP_ABS: return launch_eltwise<MI355X_OP_ABS>(A, B, C, m, st);
         default: return set_error(MI355X_ERR_INVALID_ARGUMENT, "eltwise: unknown op %d", op);
     }
 }

@@ -52,6 +52,14 @@ __device__ __forceinline__ V program_op(int op, V a, V b) {
         case MI355X_OP_GELU: return L::map([](float x, float) { return gelu_erf(x); }, a, b);
         case MI355X_OP_ERF: return L::map([](float x, float) { return erff(x); }, a, b);
         case MI355X_OP_SQRT: return L::map([](float x, float) { return sqrtf(x); }, a, b);
+        case MI355X_OP_LOG: return L::map([](float x, float) { return unary_math(MI355X_OP_LOG, x); }, a, b);
+        case MI355X_OP_TANH: return L::map([](float x, float) { return unary_math(MI355X_OP_TANH, x); }, a, b);
+        case MI355X_OP_SIGMOID: return L::map([](float x, float) { return unary_math(MI355X_OP_SIGMOID, x); }, a, b);
+        case MI355X_OP_SOFTPLUS: return L::map([](float x, float) { return unary_math(MI355X_OP_SOFTPLUS, x); }, a, b);
+        case MI355X_OP_RECIPROCAL: return L::map([](float x, float) { return unary_math(MI355X_OP_RECIPROCAL, x); }, a, b);
+        case MI355X_OP_EXP: return L::map([](float x, float) { return unary_math(MI355X_OP_EXP, x); }, a, b);
+        case MI355X_OP_NEG: return L::map([](float x, float) { return unary_math(MI355X_OP_NEG, x); }, a, b);
+        case MI355X_OP_ABS: return L::map([](float x, float) { return unary_math(MI355X_OP_ABS, x); }, a, b);
         default: return a;  // MI355X_OP_COPY
     }
 }
@@ -158,7 +166,7 @@ extern "C" int mi355x_eltwise_program_f32(const float* const* tensors, int n_ten
     uint32_t max_reg = 0;
     for (int pc = 0; pc < n_instr; ++pc) {
         const uint32_t ins = program[pc], op = ins & 255u, dst = (ins >> 8) & 255u;
-        const bool known = op <= MI355X_OP_POW || (op >= MI355X_OP_RELU && op <= MI355X_OP_COPY);
+        const bool known = op <= MI355X_OP_POW || (op >= MI355X_OP_RELU && op <= MI355X_OP_LAST);
         MI355X_REQUIRE(known && dst < 8, "eltwise_program: instruction %d (0x%08x) has an unknown op or register", pc, ins);
         const uint32_t operands[2] = {(ins >> 16) & 255u, ins >> 24};
         for (int k = 0; k < (op <= MI355X_OP_POW ? 2 : 1); ++k) {

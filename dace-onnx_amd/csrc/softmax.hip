@@ -1,9 +1,11 @@
-// ONNX Softmax, fp32, one pass over HBM.
+// ONNX Softmax and LogSoftmax, fp32, one pass over HBM.
 //
 // The reference expansion (daceml/onnx/op_implementations/pure_implementations.py:346-366)
 // runs max, subtract, exp, sum and divide as five maps with three full-size
 // temporaries. Here a row lives in registers between the read and the write,
 // so HBM traffic is the algorithmic minimum: one read and one write per element.
+// LogSoftmax (PureLogSoftmax, :594-616: (x - max) - log(sum(exp(x - max)))) is the same
+// kernels with a different last step (template parameter LOG).
 //
 // Kernels:
 //   softmax_rows_reg<L, NV, UNR>  last axis, cols % 4 == 0, cols <= L*4*NV.
@@ -33,7 +35,7 @@ __device__ __forceinline__ float group_max(float v) {
     else return wave_max(v);
 }
 
-template <int L, int NV, int UNR>
+template <int L, int NV, int UNR, bool LOG>
 __global__ __launch_bounds__(256) void softmax_rows_reg(const float* __restrict__ X,
                                                         float* __restrict__ Y,
                                                         int64_t rows, int cols) {
@@ -71,26 +73,32 @@ __global__ __launch_bounds__(256) void softmax_rows_reg(const float* __restrict_
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             // padded lanes hold -inf: exp(-inf - m) == 0 contributes nothing
-            v[u][j].x = expf(v[u][j].x - m);
-            v[u][j].y = expf(v[u][j].y - m);
-            v[u][j].z = expf(v[u][j].z - m);
-            v[u][j].w = expf(v[u][j].w - m);
-            s += (v[u][j].x + v[u][j].y) + (v[u][j].z + v[u][j].w);
+            if constexpr (LOG) {
+                v[u][j] = v[u][j] - m;   // kept for the result; the exponentials only feed the sum
+                s += (expf(v[u][j].x) + expf(v[u][j].y)) + (expf(v[u][j].z) + expf(v[u][j].w));
+            } else {
+                v[u][j].x = expf(v[u][j].x - m);
+                v[u][j].y = expf(v[u][j].y - m);
+                v[u][j].z = expf(v[u][j].z - m);
+                v[u][j].w = expf(v[u][j].w - m);
+                s += (v[u][j].x + v[u][j].y) + (v[u][j].z + v[u][j].w);
+            }
         }
         s = group_sum<L>(s);
-        const float inv = 1.0f / s;
+        const float inv = 1.0f / s, log_s = LOG ? logf(s) : 0.0f;
         f32x4* dst = reinterpret_cast<f32x4*>(Y + row * cols);
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int c4 = lane + j * L;
             if (row < rows && c4 < cols4) {
-                f32x4 o = v[u][j] * inv;
+                f32x4 o = LOG ? v[u][j] - log_s : v[u][j] * inv;
                 __builtin_nontemporal_store(o, dst + c4);
             }
         }
     }
 }
 
+template <bool LOG>
 __global__ __launch_bounds__(256) void softmax_rows_loop(const float* __restrict__ X,
                                                          float* __restrict__ Y,
                                                          int64_t rows, int64_t cols) {
@@ -105,10 +113,11 @@ __global__ __launch_bounds__(256) void softmax_rows_loop(const float* __restrict
     float s = 0.0f;
     for (int64_t c = lane; c < cols; c += WAVE) s += expf(x[c] - m);
     s = wave_sum(s);
-    const float inv = 1.0f / s;
-    for (int64_t c = lane; c < cols; c += WAVE) y[c] = expf(x[c] - m) * inv;
+    const float inv = 1.0f / s, log_s = LOG ? logf(s) : 0.0f;
+    for (int64_t c = lane; c < cols; c += WAVE) y[c] = LOG ? (x[c] - m) - log_s : expf(x[c] - m) * inv;
 }
 
+template <bool LOG>
 __global__ __launch_bounds__(256) void softmax_strided(const float* __restrict__ X,
                                                        float* __restrict__ Y,
                                                        int64_t outer, int64_t axis_len,
@@ -130,36 +139,34 @@ __global__ __launch_bounds__(256) void softmax_strided(const float* __restrict__
         for (int u = 0; u < 8; ++u) s[u] += (double)expf(x[(a + u) * inner] - m);
     }
     for (int u = 0; a < axis_len; ++a, ++u) s[u] += (double)expf(x[a * inner] - m);
-    const float inv = (float)(1.0 / (((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]))));
-    for (a = 0; a < axis_len; ++a) y[a * inner] = expf(x[a * inner] - m) * inv;
+    const double total = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+    const float inv = (float)(1.0 / total), log_s = LOG ? (float)log(total) : 0.0f;
+    for (a = 0; a < axis_len; ++a) y[a * inner] = LOG ? (x[a * inner] - m) - log_s : expf(x[a * inner] - m) * inv;
 }
 
-template <int L, int NV, int UNR>
+template <int L, int NV, int UNR, bool LOG>
 static void launch_reg(const float* X, float* Y, int64_t rows, int cols, hipStream_t st) {
     constexpr int rows_per_block = (256 / L) * UNR;
     const int64_t blocks = ceil_div(rows, rows_per_block);
-    hipLaunchKernelGGL((softmax_rows_reg<L, NV, UNR>), dim3((unsigned)blocks), dim3(256), 0, st,
+    hipLaunchKernelGGL((softmax_rows_reg<L, NV, UNR, LOG>), dim3((unsigned)blocks), dim3(256), 0, st,
                        X, Y, rows, cols);
 }
 
 // Pick the unroll so that a full launch is a whole number of blocks per CU
 // where possible (12288 rows of 128 -> 512 blocks of 24 rows on 256 CUs).
-template <int L, int NV>
+template <int L, int NV, bool LOG>
 static void launch_reg_unr(const float* X, float* Y, int64_t rows, int cols, hipStream_t st) {
     constexpr int groups = 256 / L;
     if (NV <= 2 && rows % (groups * 3) == 0 && rows >= (int64_t)groups * 3 * 256)
-        launch_reg<L, NV, (NV <= 2 ? 3 : 1)>(X, Y, rows, cols, st);
+        launch_reg<L, NV, (NV <= 2 ? 3 : 1), LOG>(X, Y, rows, cols, st);
     else if (NV <= 2 && rows >= (int64_t)groups * 2 * 512)
-        launch_reg<L, NV, (NV <= 2 ? 2 : 1)>(X, Y, rows, cols, st);
+        launch_reg<L, NV, (NV <= 2 ? 2 : 1), LOG>(X, Y, rows, cols, st);
     else
-        launch_reg<L, NV, 1>(X, Y, rows, cols, st);
+        launch_reg<L, NV, 1, LOG>(X, Y, rows, cols, st);
 }
 
-}  // namespace mi355x
-
-extern "C" int mi355x_softmax_f32(const float* X, float* Y, int64_t outer, int64_t axis_len,
-                                  int64_t inner, void* stream) {
-    using namespace mi355x;
+template <bool LOG>
+static int softmax_dispatch(const float* X, float* Y, int64_t outer, int64_t axis_len, int64_t inner, void* stream) {
     MI355X_REQUIRE(outer >= 0 && axis_len >= 0 && inner >= 0,
                    "softmax: negative extent (outer=%lld axis_len=%lld inner=%lld)",
                    (long long)outer, (long long)axis_len, (long long)inner);
@@ -172,20 +179,32 @@ extern "C" int mi355x_softmax_f32(const float* X, float* Y, int64_t outer, int64
         MI355X_REQUIRE(rows < ((int64_t)1 << 31), "softmax: too many rows (%lld)", (long long)rows);
         const bool vec_ok = (cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(X) & 15) == 0) &&
                             ((reinterpret_cast<uintptr_t>(Y) & 15) == 0);
-        if (vec_ok && cols <= 64) launch_reg_unr<16, 1>(X, Y, rows, (int)cols, st);
-        else if (vec_ok && cols <= 128) launch_reg_unr<32, 1>(X, Y, rows, (int)cols, st);
-        else if (vec_ok && cols <= 256) launch_reg_unr<64, 1>(X, Y, rows, (int)cols, st);
-        else if (vec_ok && cols <= 512) launch_reg_unr<64, 2>(X, Y, rows, (int)cols, st);
-        else if (vec_ok && cols <= 1024) launch_reg_unr<64, 4>(X, Y, rows, (int)cols, st);
-        else if (vec_ok && cols <= 2048) launch_reg_unr<64, 8>(X, Y, rows, (int)cols, st);
+        if (vec_ok && cols <= 64) launch_reg_unr<16, 1, LOG>(X, Y, rows, (int)cols, st);
+        else if (vec_ok && cols <= 128) launch_reg_unr<32, 1, LOG>(X, Y, rows, (int)cols, st);
+        else if (vec_ok && cols <= 256) launch_reg_unr<64, 1, LOG>(X, Y, rows, (int)cols, st);
+        else if (vec_ok && cols <= 512) launch_reg_unr<64, 2, LOG>(X, Y, rows, (int)cols, st);
+        else if (vec_ok && cols <= 1024) launch_reg_unr<64, 4, LOG>(X, Y, rows, (int)cols, st);
+        else if (vec_ok && cols <= 2048) launch_reg_unr<64, 8, LOG>(X, Y, rows, (int)cols, st);
         else
-            hipLaunchKernelGGL(softmax_rows_loop, dim3((unsigned)ceil_div(rows, 256 / WAVE)),
+            hipLaunchKernelGGL(softmax_rows_loop<LOG>, dim3((unsigned)ceil_div(rows, 256 / WAVE)),
                                dim3(256), 0, st, X, Y, rows, cols);
         return check_launch("softmax_rows");
     }
     const int64_t n = outer * inner;
     MI355X_REQUIRE(ceil_div(n, 256) < ((int64_t)1 << 31), "softmax: grid too large");
-    hipLaunchKernelGGL(softmax_strided, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, X, Y,
+    hipLaunchKernelGGL(softmax_strided<LOG>, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, X, Y,
                        outer, axis_len, inner);
     return check_launch("softmax_strided");
+}
+
+}  // namespace mi355x
+
+extern "C" int mi355x_softmax_f32(const float* X, float* Y, int64_t outer, int64_t axis_len,
+                                  int64_t inner, void* stream) {
+    return mi355x::softmax_dispatch<false>(X, Y, outer, axis_len, inner, stream);
+}
+
+extern "C" int mi355x_log_softmax_f32(const float* X, float* Y, int64_t outer, int64_t axis_len,
+                                      int64_t inner, void* stream) {
+    return mi355x::softmax_dispatch<true>(X, Y, outer, axis_len, inner, stream);
 }

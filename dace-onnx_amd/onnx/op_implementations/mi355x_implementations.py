@@ -408,6 +408,21 @@ class MI355XSoftmax(ONNXForward):
                                     [Ptr("input"), Ptr("output"), outer, axis_len, inner, Stream()])
 
 
+@op_implementation(op="LogSoftmax", name=IMPLEMENTATION_NAME)
+class MI355XLogSoftmax(ONNXForward):
+    """LogSoftmax along ``node.axis`` only, as PureLogSoftmax computes it (:594-616), in one pass."""
+
+    forward_can_be_applied = MI355XSoftmax.forward_can_be_applied
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "input")
+        axis = node.axis % len(X.shape)
+        outer, axis_len, inner = prod(X.shape[:axis]), X.shape[axis], prod(X.shape[axis + 1:])
+        return kernel_call_for_node(node, state, "mi355x_log_softmax_f32",
+                                    [Ptr("input"), Ptr("output"), outer, axis_len, inner, Stream()])
+
+
 @op_implementation(op="FusedAttention", name=IMPLEMENTATION_NAME)
 class MI355XFusedAttention(ONNXForward):
     """``softmax(scale * Q K^T) V`` in one launch; scores stay in registers. The
@@ -469,40 +484,54 @@ class MI355XFusedAttention(ONNXForward):
             float(node.scale if node.scale is not None else 1.0), Stream()])
 
 
-@op_implementation(op="ReduceMean", name=IMPLEMENTATION_NAME)
-class MI355XReduceMean(ONNXForward):
-    """Mean over ``axes`` (attribute form, opset < 18) when they are adjacent, which
-    makes them one axis of the product length (PureReduceMean, :97-109)."""
+def _reduce_split(node, X):
+    """(outer, axis_len, inner, reduced axes) when the reduced axes are adjacent -- which makes them one axis
+    of the product length -- or None."""
+    rank = len(X.shape)
+    axes = sorted(a % rank for a in node.axes) if node.axes is not None else list(range(rank))
+    if not axes or axes != list(range(axes[0], axes[-1] + 1)) or any(not -rank <= a < rank for a in (node.axes or [])):
+        return None
+    return prod(X.shape[:axes[0]]), prod(X.shape[axes[0]:axes[-1] + 1]), prod(X.shape[axes[-1] + 1:]), axes
 
-    @staticmethod
-    def _split(node, X):
-        """(outer, axis_len, inner, reduced axes) or None."""
-        rank = len(X.shape)
-        axes = sorted(a % rank for a in node.axes) if node.axes is not None else list(range(rank))
-        if not axes or axes != list(range(axes[0], axes[-1] + 1)) or any(not -rank <= a < rank for a in (node.axes or [])):
-            return None
-        return prod(X.shape[:axes[0]]), prod(X.shape[axes[0]:axes[-1] + 1]), prod(X.shape[axes[-1] + 1:]), axes
 
-    @staticmethod
-    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
-        X = in_desc_with_name(node, state, sdfg, "data")
-        Y = out_desc_with_name(node, state, sdfg, "reduced")
-        if not _is_f32(X, Y) or not _contig(X, Y) or len(X.shape) < 1:
-            return False
-        split = MI355XReduceMean._split(node, X)
-        if split is None or split[1] < 1:
-            return False
-        keep = node.keepdims is None or bool(node.keepdims)
-        want = [1 if d in split[3] else e for d, e in enumerate(X.shape)] if keep else \
-            [e for d, e in enumerate(X.shape) if d not in split[3]]
-        return [e for e in Y.shape if e != 1] == [e for e in want if e != 1] and Y.total_size == split[0] * split[2]
+def _reduce_impl(op_name, kind, cite):
+    @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
+    class Impl(ONNXForward):
+        __doc__ = (f"{op_name} over ``axes`` (attribute form, opset < 13 / 18) when they are adjacent "
+                   f"({cite}).")
 
-    @staticmethod
-    def forward(node, state: SDFGState, sdfg: SDFG):
-        X = in_desc_with_name(node, state, sdfg, "data")
-        outer, axis_len, inner, _ = MI355XReduceMean._split(node, X)
-        return kernel_call_for_node(node, state, "mi355x_reduce_mean_f32",
-                                    [Ptr("data"), Ptr("reduced"), outer, axis_len, inner, Stream()])
+        @staticmethod
+        def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+            X = in_desc_with_name(node, state, sdfg, "data")
+            Y = out_desc_with_name(node, state, sdfg, "reduced")
+            if not _is_f32(X, Y) or not _contig(X, Y) or len(X.shape) < 1:
+                return False
+            split = _reduce_split(node, X)
+            if split is None or split[1] < 1:
+                return False
+            keep = node.keepdims is None or bool(node.keepdims)
+            want = [1 if d in split[3] else e for d, e in enumerate(X.shape)] if keep else \
+                [e for d, e in enumerate(X.shape) if d not in split[3]]
+            return [e for e in Y.shape if e != 1] == [e for e in want if e != 1] and Y.total_size == split[0] * split[2]
+
+        @staticmethod
+        def forward(node, state: SDFGState, sdfg: SDFG):
+            X = in_desc_with_name(node, state, sdfg, "data")
+            outer, axis_len, inner, _ = _reduce_split(node, X)
+            if kind == _lib.REDUCE_MEAN:
+                return kernel_call_for_node(node, state, "mi355x_reduce_mean_f32",
+                                            [Ptr("data"), Ptr("reduced"), outer, axis_len, inner, Stream()])
+            return kernel_call_for_node(node, state, "mi355x_reduce_f32",
+                                        [kind, Ptr("data"), Ptr("reduced"), outer, axis_len, inner, Stream()])
+
+    Impl.__name__ = Impl.__qualname__ = "MI355X" + op_name
+    return Impl
+
+
+MI355XReduceMean = _reduce_impl("ReduceMean", _lib.REDUCE_MEAN, "PureReduceMean, :97-109")
+MI355XReduceSum = _reduce_impl("ReduceSum", _lib.REDUCE_SUM, "PureReduceSum, :301-313")
+MI355XReduceMax = _reduce_impl("ReduceMax", _lib.REDUCE_MAX, "PureReduceMax, :316-328")
+MI355XReduceMin = _reduce_impl("ReduceMin", _lib.REDUCE_MIN, "PureReduceMin, :331-343")
 
 
 @op_implementation(op="LayerNormalization", name=IMPLEMENTATION_NAME)
@@ -607,6 +636,16 @@ MI355XGelu = _unary_impl("Gelu", _lib.OP_GELU, "X", "Y",
                          extra_check=lambda node: (node.approximate or "none") == "none")
 MI355XErf = _unary_impl("Erf", _lib.OP_ERF, "input", "output")
 MI355XSqrt = _unary_impl("Sqrt", _lib.OP_SQRT, "X", "Y")
+# PureLog (:23-38), Tanh (:296-298), PureSigmoid (:701-712), Softplus (:696-698), PureReciprocal (:275-293);
+# Exp, Neg and Abs have no pure expansion in the reference
+MI355XLog = _unary_impl("Log", _lib.OP_LOG, "input", "output")
+MI355XTanh = _unary_impl("Tanh", _lib.OP_TANH, "input", "output")
+MI355XExp = _unary_impl("Exp", _lib.OP_EXP, "input", "output")
+MI355XSigmoid = _unary_impl("Sigmoid", _lib.OP_SIGMOID, "X", "Y")
+MI355XSoftplus = _unary_impl("Softplus", _lib.OP_SOFTPLUS, "X", "Y")
+MI355XReciprocal = _unary_impl("Reciprocal", _lib.OP_RECIPROCAL, "X", "Y")
+MI355XNeg = _unary_impl("Neg", _lib.OP_NEG, "X", "Y")
+MI355XAbs = _unary_impl("Abs", _lib.OP_ABS, "X", "Y")
 
 
 # ------------------------------------------------------------------------------------
@@ -721,3 +760,37 @@ class MI355XFusedElementwise(ONNXForward):
         return kernel_call_for_node(node, state, "mi355x_eltwise_program_f32", [
             PtrArray(tensors), len(tensors), PtrArray(vectors), len(vectors), Ptr("Y"), int(Y.total_size),
             int(Y.shape[-1]) if Y.shape else 1, U32Array(node.program), len(node.program), F32Array(imms), len(imms), Stream()])
+
+
+
+@op_implementation(op="Sum", name=IMPLEMENTATION_NAME)
+class MI355XSum(ONNXForward):
+    """Sum of up to four tensors of one shape -- the case PureSum accepts (:529-591, all shapes equal to the
+    output's) -- as one launch of the program kernel: every input read once, no intermediate sums."""
+
+    @staticmethod
+    def _inputs(node):
+        return sorted((c for c in node.in_connectors if c.startswith("data_0__")), key=lambda c: int(c[len("data_0__"):]))
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        conns = MI355XSum._inputs(node)
+        Y = out_desc_with_name(node, state, sdfg, "sum")
+        if not 1 <= len(conns) <= _lib.PROGRAM_MAX_TENSORS or not _is_f32(Y) or not _contig(Y):
+            return False
+        descs = [in_desc_with_name(node, state, sdfg, c) for c in conns]
+        return all(_is_f32(d) and _contig(d) and tuple(d.shape) == tuple(Y.shape) for d in descs)
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        conns = MI355XSum._inputs(node)
+        Y = out_desc_with_name(node, state, sdfg, "sum")
+        tensor = lambda i: (_lib.PROGRAM_TENSOR << 6) | i
+        if len(conns) == 1:
+            program = [_lib.OP_COPY | tensor(0) << 16]
+        else:   # r0 = t0 + t1; r0 = r0 + t2; ...
+            program = [_lib.OP_ADD | tensor(0) << 16 | tensor(1) << 24]
+            program += [_lib.OP_ADD | (_lib.PROGRAM_REG << 6) << 16 | tensor(i) << 24 for i in range(2, len(conns))]
+        return kernel_call_for_node(node, state, "mi355x_eltwise_program_f32", [
+            PtrArray(conns), len(conns), PtrArray([]), 0, Ptr("sum"), int(Y.total_size),
+            int(Y.shape[-1]) if Y.shape else 1, U32Array(program), len(program), F32Array([]), 0, Stream()])

@@ -126,6 +126,10 @@ SCHEMAS: typing.List[ONNXSchema] = [
     _unary("Gelu", 20, "X", "Y", attributes=[ONNXAttribute("approximate", _A.String, "none")]),
     _unary("Erf", 9, "input", "output", types=_NUMERIC),
     _unary("Sqrt", 6, "X", "Y"),
+    _unary("Log", 6, "input", "output"), _unary("Tanh", 6, "input", "output"), _unary("Exp", 6, "input", "output"),
+    _unary("Sigmoid", 6, "X", "Y"), _unary("Softplus", 1, "X", "Y"), _unary("Reciprocal", 6, "X", "Y"),
+    _unary("Neg", 6, "X", "Y", types=_FLOATS + [dace.int32, dace.int64, dace.int8, dace.int16]),
+    _unary("Abs", 6, "X", "Y", types=_NUMERIC),
     ONNXSchema("Reshape", 5, [ONNXParameter("data", "T"), ONNXParameter("shape", "tensor(int64)")],
                [ONNXParameter("reshaped", "T")], (),
                [ONNXTypeConstraint("T", _ANY), ONNXTypeConstraint("tensor(int64)", [dace.int64])]),
@@ -150,9 +154,16 @@ SCHEMAS: typing.List[ONNXSchema] = [
                "Y = program(X__0, X__1, ...): instructions, immediates and operand kinds as in mi355x_eltwise_program_f32."),
     ONNXSchema("Pow", 12, [ONNXParameter("X", "T"), ONNXParameter("Y", "T1")], [ONNXParameter("Z", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64]), ONNXTypeConstraint("T1", _NUMERIC)]),
-    ONNXSchema("ReduceMean", 11, [ONNXParameter("data", "T")], [ONNXParameter("reduced", "T")],
+] + [
+    ONNXSchema(name, 11, [ONNXParameter("data", "T")], [ONNXParameter("reduced", "T")],
                [ONNXAttribute("axes", _A.Ints), ONNXAttribute("keepdims", _A.Int, 1)],
-               [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64])]),
+               [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64])])
+    for name in ("ReduceMean", "ReduceSum", "ReduceMax", "ReduceMin")
+] + [
+    _unary("LogSoftmax", 11, "input", "output", attributes=[ONNXAttribute("axis", _A.Int, 1)],
+           doc="Log of the softmax along `axis`."),
+    ONNXSchema("Sum", 8, [ONNXParameter("data_0", "T", ONNXParameterType.Variadic)], [ONNXParameter("sum", "T")], (),
+               [ONNXTypeConstraint("T", _FLOATS)], "Elementwise sum of the inputs."),
 ]
 
 SCHEMAS_BY_NAME = {s.name: s for s in SCHEMAS}

@@ -37,7 +37,8 @@ def _infer_node(node, shapes, types, constants):
         raise ShapeInferenceError(f"{op} node '{node.name}': no shape for input(s) {missing}")
     if op in ("Add", "Sub", "Mul", "Div", "Pow"):
         return [(tuple(np.broadcast_shapes(ins[0], ins[1])), tys[0])]
-    if op in ("Relu", "Gelu", "Erf", "Sqrt", "Softmax", "Identity", "Tanh", "Sigmoid"):
+    if op in ("Relu", "Gelu", "Erf", "Sqrt", "Softmax", "LogSoftmax", "Identity", "Tanh", "Sigmoid", "Log", "Exp", "Softplus",
+              "Reciprocal", "Neg", "Abs"):
         return [(ins[0], tys[0])]
     if op == "LayerNormalization":
         return [(ins[0], tys[0])]
@@ -98,7 +99,9 @@ def _infer_node(node, shapes, types, constants):
     if op == "Flatten":
         axis = a.get("axis", 1) % (len(ins[0]) + 1) if a.get("axis", 1) < 0 else a.get("axis", 1)
         return [((int(np.prod(ins[0][:axis])) if axis else 1, int(np.prod(ins[0][axis:]))), tys[0])]
-    if op == "ReduceMean":
+    if op == "Sum":
+        return [(tuple(np.broadcast_shapes(*ins)), tys[0])]
+    if op in ("ReduceMean", "ReduceSum", "ReduceMax", "ReduceMin"):
         axes = a.get("axes") or list(range(len(ins[0])))
         axes = [ax % len(ins[0]) for ax in axes]
         keep = a.get("keepdims", 1)

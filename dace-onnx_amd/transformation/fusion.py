@@ -937,21 +937,22 @@ def _fuse_shared_input_matmuls(sdfg: SDFG, state: SDFGState) -> int:
 
 
 _EW_BINARY = {"Add": _lib.OP_ADD, "Sub": _lib.OP_SUB, "Mul": _lib.OP_MUL, "Div": _lib.OP_DIV, "Pow": _lib.OP_POW}
-_EW_UNARY = {"Relu": _lib.OP_RELU, "Gelu": _lib.OP_GELU, "Erf": _lib.OP_ERF, "Sqrt": _lib.OP_SQRT, "Identity": _lib.OP_COPY}
-
-
-class _ProgramTooLarge(Exception):
-    pass
+_EW_UNARY = {"Relu": _lib.OP_RELU, "Gelu": _lib.OP_GELU, "Erf": _lib.OP_ERF, "Sqrt": _lib.OP_SQRT, "Identity": _lib.OP_COPY,
+             "Log": _lib.OP_LOG, "Tanh": _lib.OP_TANH, "Sigmoid": _lib.OP_SIGMOID, "Softplus": _lib.OP_SOFTPLUS,
+             "Reciprocal": _lib.OP_RECIPROCAL, "Exp": _lib.OP_EXP, "Neg": _lib.OP_NEG, "Abs": _lib.OP_ABS}
 
 
 def _fuse_elementwise(sdfg: SDFG, state: SDFGState) -> int:
-    """Groups of elementwise nodes (Add, Sub, Mul, Div, Pow, Relu, Gelu, Erf, Sqrt, Identity) whose
-    intermediate results have one reader become one ``FusedElementwise`` node: a short program for
-    ``mi355x_eltwise_program_f32`` in which every tensor operand is read once and only the final result is
-    written -- what the reference leaves to DaCe's map / tasklet fusion after expansion
-    (``daceml/transformation/tasklet_fusion.py``). A group is grown backwards from its last node; an operand
-    is another member's result, a tensor of the result's shape, a vector along the last axis, or a scalar
-    constant. Runs last, on whatever the GEMM / Conv epilogue folds and the pattern rewrites left over."""
+    """Groups of elementwise nodes (Add, Sub, Mul, Div, Pow and the unary maps of ``_EW_UNARY``) whose
+    intermediate results are read only inside the group become one ``FusedElementwise`` node: a short
+    program for ``mi355x_eltwise_program_f32`` in which every tensor operand is read once and only the final
+    result is written -- what the reference leaves to DaCe's map / tasklet fusion after expansion
+    (``daceml/transformation/tasklet_fusion.py``). A group is grown backwards from its last node: a producer
+    joins when every reader of its result already belongs to the group (so ``g * sigmoid(g)`` keeps ``g`` in
+    a register for both readers). An operand is another member's result, a tensor of the result's shape, a
+    vector along the last axis, or a scalar constant. When a group does not fit the kernel's limits
+    (instructions, registers, operands), members are dropped from its input side until it does. Runs last,
+    on whatever the GEMM / Conv epilogue folds and the pattern rewrites left over."""
     from ..onnx.nodes.onnx_op import get_onnx_node
 
     def fusable(n):
@@ -968,10 +969,83 @@ def _fuse_elementwise(sdfg: SDFG, state: SDFGState) -> int:
     def f32_contiguous(desc):
         return desc.dtype.name == "float32" and desc.is_contiguous()
 
+    def readers(acc):
+        """Nodes reading the transient behind ``acc`` (one entry per edge), or None when the value is visible
+        outside the state's dataflow (not transient, written more than once, or accessed elsewhere)."""
+        desc = sdfg.arrays[acc.data]
+        if not desc.transient or len(state.in_edges(acc)) != 1:
+            return None
+        if any(isinstance(n, AccessNode) and n is not acc and n.data == acc.data for n in state.nodes()):
+            return None
+        return [e.dst for e in state.out_edges(acc)]
+
+    def result_of(n):
+        return io_edges(n)[1].dst
+
+    def try_program(members, shape):
+        """(program, tensors, vectors, immediates) for ``members`` (operands before their readers), or None when an
+        operand cannot be expressed or a limit of the kernel is exceeded."""
+        produced = {result_of(m).data: m for m in members}
+        uses_left = {}
+        for m in members:
+            for e in io_edges(m)[0]:
+                if e.src.data in produced:
+                    uses_left[e.src.data] = uses_left.get(e.src.data, 0) + 1
+        tensors, vectors, imms, program, reg_of = [], [], [], [], {}
+        free_regs = list(range(8))
+        for m in members:
+            encoded = []
+            for e in io_edges(m)[0]:
+                name = e.src.data
+                desc = sdfg.arrays[name]
+                const = _constant_value(sdfg, name) if not state.in_edges(e.src) else None
+                if name in produced:
+                    encoded.append((_lib.PROGRAM_REG << 6) | reg_of[name])
+                elif const is not None and const.size == 1 and const.dtype == np.float32:
+                    v = float(const.reshape(-1)[0])
+                    if v not in imms:
+                        imms.append(v)
+                    encoded.append((_lib.PROGRAM_IMMEDIATE << 6) | imms.index(v))
+                elif not f32_contiguous(desc):
+                    return None
+                elif tuple(desc.shape) == shape:
+                    if name not in tensors:
+                        tensors.append(name)
+                    encoded.append((_lib.PROGRAM_TENSOR << 6) | tensors.index(name))
+                elif desc.total_size == shape[-1] and desc.shape and desc.shape[-1] == shape[-1]:
+                    if name not in vectors:
+                        vectors.append(name)
+                    encoded.append((_lib.PROGRAM_VECTOR << 6) | vectors.index(name))
+                else:
+                    return None     # a broadcast this kernel does not do
+            for e in io_edges(m)[0]:     # operands read for the last time give their register back
+                name = e.src.data
+                if name in produced:
+                    uses_left[name] -= 1
+                    if uses_left[name] == 0:
+                        free_regs.append(reg_of[name])
+            if not free_regs:
+                return None
+            dst = min(free_regs)
+            free_regs.remove(dst)
+            reg_of[result_of(m).data] = dst
+            a = encoded[0]
+            b = encoded[1] if len(encoded) > 1 else 0
+            if _is_op(m, "Pow") and (b >> 6) == _lib.PROGRAM_IMMEDIATE and imms[b & 63] == 2.0:
+                op, b = _lib.OP_MUL, a
+            else:
+                op = _EW_BINARY.get(m.schema.name, _EW_UNARY.get(m.schema.name))
+            program.append(op | (dst << 8) | (a << 16) | (b << 24))
+        if len(program) > _lib.PROGRAM_MAX_INSTR or len(tensors) > _lib.PROGRAM_MAX_TENSORS or \
+                len(vectors) > _lib.PROGRAM_MAX_VECTORS or len(imms) > _lib.PROGRAM_MAX_IMM:
+            return None
+        return program, tensors, vectors, imms
+
     done = set()
     fused = 0
-    for final in reversed(list(state.topological_nodes())):
-        if final in done or not fusable(final):
+    order = {n: i for i, n in enumerate(state.topological_nodes())}
+    for final in sorted((n for n in order if fusable(n)), key=lambda n: -order[n]):
+        if final in done or final not in state.nodes():
             continue
         ins, out_e = io_edges(final)
         if out_e is None or not isinstance(out_e.dst, AccessNode) or any(e is None for e in ins):
@@ -979,73 +1053,53 @@ def _fuse_elementwise(sdfg: SDFG, state: SDFGState) -> int:
         shape = tuple(sdfg.arrays[out_e.dst.data].shape)
         if not shape or not f32_contiguous(sdfg.arrays[out_e.dst.data]):
             continue
-        members, tensors, vectors, imms, program = [], [], [], [], []
-        free_regs = list(range(8))
 
-        def operand(edge):
-            """Encoded operand for the value on ``edge``; absorbs its producer when it can join the group."""
-            acc = edge.src
-            desc = sdfg.arrays[acc.data]
-            const = _constant_value(sdfg, acc.data) if not state.in_edges(acc) else None
-            if const is not None and const.size == 1 and const.dtype == np.float32:
-                v = float(const.reshape(-1)[0])
-                if v not in imms:
-                    imms.append(v)
-                return (_lib.PROGRAM_IMMEDIATE << 6) | imms.index(v), None
-            prod = _producer(state, acc)
-            if prod is not None and fusable(prod.src) and prod.src not in done and tuple(desc.shape) == shape \
-                    and f32_contiguous(desc) and _single_consumer(sdfg, state, acc) is not None:
-                p_ins, _ = io_edges(prod.src)
-                if all(e is not None for e in p_ins):
-                    # tentative: if the producer (or something it needs) does not fit, it stays outside and
-                    # its result is read as a tensor
-                    snapshot = (len(members), len(program), list(free_regs), len(tensors), len(vectors), len(imms))
-                    try:
-                        reg = emit(prod.src, p_ins)
-                        return (_lib.PROGRAM_REG << 6) | reg, reg
-                    except _ProgramTooLarge:
-                        del members[snapshot[0]:], program[snapshot[1]:], tensors[snapshot[3]:], vectors[snapshot[4]:]
-                        del imms[snapshot[5]:]
-                        free_regs[:] = snapshot[2]
-            if not f32_contiguous(desc):
-                raise _ProgramTooLarge()
-            if tuple(desc.shape) == shape:
-                if acc.data not in tensors:
-                    tensors.append(acc.data)
-                return (_lib.PROGRAM_TENSOR << 6) | tensors.index(acc.data), None
-            if desc.total_size == shape[-1] and desc.shape and desc.shape[-1] == shape[-1]:
-                if acc.data not in vectors:
-                    vectors.append(acc.data)
-                return (_lib.PROGRAM_VECTOR << 6) | vectors.index(acc.data), None
-            raise _ProgramTooLarge()     # a broadcast this kernel does not do
+        def closure(excluded):
+            """Members reachable backwards from ``final`` whose results are read only by members."""
+            group = {final}
+            changed = True
+            while changed:
+                changed = False
+                for m in list(group):
+                    for e in io_edges(m)[0]:
+                        prod = _producer(state, e.src)
+                        if prod is None or prod.src in group or prod.src in excluded or prod.src in done \
+                                or not fusable(prod.src):
+                            continue
+                        desc = sdfg.arrays[e.src.data]
+                        p_ins, p_out = io_edges(prod.src)
+                        rd = readers(e.src)
+                        if tuple(desc.shape) == shape and f32_contiguous(desc) and rd is not None and \
+                                all(r in group for r in rd) and all(pe is not None for pe in p_ins) and p_out is not None:
+                            group.add(prod.src)
+                            changed = True
+            # operands first, depth first from the last node: a valid order that keeps few values alive at once
+            ordered, seen = [], set()
 
-        def emit(n, in_edges):
-            encoded = [operand(e) for e in in_edges]
-            for _, reg in encoded:
-                if reg is not None:
-                    free_regs.append(reg)       # an intermediate has exactly one reader: this instruction
-            if not free_regs:
-                raise _ProgramTooLarge()
-            dst = min(free_regs)
-            free_regs.remove(dst)
-            a = encoded[0][0]
-            b = encoded[1][0] if len(encoded) > 1 else 0
-            if _is_op(n, "Pow") and (b >> 6) == _lib.PROGRAM_IMMEDIATE and imms[b & 63] == 2.0:
-                op, b = _lib.OP_MUL, a
-            else:
-                op = _EW_BINARY.get(n.schema.name, _EW_UNARY.get(n.schema.name))
-            program.append(op | (dst << 8) | (a << 16) | (b << 24))
-            members.append(n)
-            if len(program) > _lib.PROGRAM_MAX_INSTR or len(tensors) > _lib.PROGRAM_MAX_TENSORS or \
-                    len(vectors) > _lib.PROGRAM_MAX_VECTORS or len(imms) > _lib.PROGRAM_MAX_IMM:
-                raise _ProgramTooLarge()
-            return dst
+            def visit(m):
+                if m in seen:
+                    return
+                seen.add(m)
+                for e in io_edges(m)[0]:
+                    prod = _producer(state, e.src)
+                    if prod is not None and prod.src in group:
+                        visit(prod.src)
+                ordered.append(m)
 
-        try:
-            emit(final, ins)
-        except _ProgramTooLarge:
+            visit(final)
+            return ordered
+
+        excluded = set()
+        members = closure(excluded)
+        built = try_program(members, shape)
+        while built is None and len(members) > 2:
+            excluded.add(members[0])     # shrink from the input side; the closure drops whatever only fed it
+            members = closure(excluded)
+            built = try_program(members, shape)
+        if built is None or len(members) < 2:
             continue
-        if len(members) < 2 or not (tensors or vectors):
+        program, tensors, vectors, imms = built
+        if not (tensors or vectors):
             continue
         # ---- rewrite
         node = get_onnx_node("FusedElementwise")(final.label + "_fused", program=list(program), immediates=list(imms),
@@ -1060,7 +1114,7 @@ def _fuse_elementwise(sdfg: SDFG, state: SDFGState) -> int:
             state.add_edge(accesses[name], None, node, f"X__{i}", sdfg.make_array_memlet(name))
         node.add_out_connector("Y")
         state.add_edge(node, "Y", out_e.dst, None, sdfg.make_array_memlet(out_e.dst.data))
-        intermediates = [_out_edge(state, m, m.schema.outputs[0].name).dst for m in members if m is not final]
+        intermediates = [result_of(m) for m in members if m is not final]
         for m in members:
             state.remove_node(m)
             done.add(m)

@@ -126,6 +126,13 @@ int mi355x_softmax_f32(const float* X, float* Y,
                        int64_t outer, int64_t axis_len, int64_t inner,
                        void* stream);
 
+/* ONNX LogSoftmax along one axis, fp32, same view of X:
+ * y = (x - max) - log(sum(exp(x - max))). Replaces the eight steps of
+ * PureLogSoftmax.forward (pure_implementations.py:594-616) with one pass. */
+int mi355x_log_softmax_f32(const float* X, float* Y,
+                           int64_t outer, int64_t axis_len, int64_t inner,
+                           void* stream);
+
 /* Scaled-dot-product attention core, fp32, one launch:
  *   O[b0,b1] = softmax(scale * Q[b0,b1] K[b0,b1]^T, over keys) V[b0,b1]
  * Q, O are [Sq, D], K, V are [Sk, D] per (b0, b1) slice; the last dimension is
@@ -164,11 +171,27 @@ int mi355x_reduce_mean_f32(const float* X, float* Y,
                            int64_t outer, int64_t axis_len, int64_t inner,
                            void* stream);
 
+/* ONNX ReduceMean / ReduceSum / ReduceMax / ReduceMin along one axis, fp32, same
+ * view of X and Y as mi355x_reduce_mean_f32 (which is kind MI355X_REDUCE_MEAN).
+ * Replaces PureReduceSum, PureReduceMax and PureReduceMin
+ * (pure_implementations.py:301-343: np.sum / np.max / np.min over `axes`). A
+ * NaN in a reduced slice makes its maximum and minimum NaN, as numpy does. */
+#define MI355X_REDUCE_MEAN 0
+#define MI355X_REDUCE_SUM 1
+#define MI355X_REDUCE_MAX 2
+#define MI355X_REDUCE_MIN 3
+int mi355x_reduce_f32(int kind, const float* X, float* Y,
+                      int64_t outer, int64_t axis_len, int64_t inner,
+                      void* stream);
+
 /* Elementwise ops, fp32, with numpy broadcasting.
  * Replaces the one-map expansions Add/Sub/Mul/Div
  * (pure_implementations.py:77-94), PurePow (:59-74), PureRelu (:462-474),
- * PureErf (:112-127), PureSqrt (:41-56) and the Gelu decomposition
- * Div,Erf,Add,Mul,Mul.
+ * PureErf (:112-127), PureSqrt (:41-56), the Gelu decomposition
+ * Div,Erf,Add,Mul,Mul, and the unary maps PureLog (:23-38), PureReciprocal
+ * (:275-293), Tanh (:296-298), Softplus (:696-698, log(1 + exp(x)) as written
+ * there) and PureSigmoid (:701-712, 1 / (1 + exp(-x))); Exp, Neg and Abs have
+ * no pure expansion in the reference (ONNX Runtime runs them there).
  *   binary ops: C = A op B; unary ops ignore B (pass NULL).
  *   ndim <= 8; shape is the OUTPUT shape; a_strides / b_strides are element
  *   strides of each operand in the output's index space (0 on broadcast dims).
@@ -182,6 +205,16 @@ int mi355x_reduce_mean_f32(const float* X, float* Y,
 #define MI355X_OP_GELU 17
 #define MI355X_OP_ERF 18
 #define MI355X_OP_SQRT 19
+/* 20 is MI355X_OP_COPY, see the program kernel below */
+#define MI355X_OP_LOG 21
+#define MI355X_OP_TANH 22
+#define MI355X_OP_SIGMOID 23
+#define MI355X_OP_SOFTPLUS 24
+#define MI355X_OP_RECIPROCAL 25
+#define MI355X_OP_EXP 26
+#define MI355X_OP_NEG 27
+#define MI355X_OP_ABS 28
+#define MI355X_OP_LAST 28
 int mi355x_eltwise_f32(int op, const float* A, const float* B, float* C,
                        int ndim, const int64_t* shape,
                        const int64_t* a_strides, const int64_t* b_strides,

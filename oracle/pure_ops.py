@@ -174,6 +174,42 @@ def reduce_mean(data, axes, keepdims=1):
     return np.mean(data, axis=tuple(axes), keepdims=bool(keepdims)).astype(data.dtype, copy=False)
 
 
+def reduce_sum(data, axes, keepdims=1):
+    """PureReduceSum: np.sum over ``axes`` (pure_implementations.py:301-313)."""
+    return np.sum(data, axis=tuple(axes), keepdims=bool(keepdims)).astype(data.dtype, copy=False)
+
+
+def reduce_max(data, axes, keepdims=1):
+    """PureReduceMax: np.max over ``axes`` (pure_implementations.py:316-328)."""
+    return np.max(data, axis=tuple(axes), keepdims=bool(keepdims))
+
+
+def reduce_min(data, axes, keepdims=1):
+    """PureReduceMin: np.min over ``axes`` (pure_implementations.py:331-343)."""
+    return np.min(data, axis=tuple(axes), keepdims=bool(keepdims))
+
+
+def log_softmax(X, axis=-1):
+    """PureLogSoftmax, step by step as the reference writes it (pure_implementations.py:594-616):
+    max, subtract, exp, sum, log, subtract."""
+    reduced_shape = list(X.shape)
+    reduced_shape[axis] = 1
+    max_keepdims = np.reshape(np.max(X, axis=axis), reduced_shape)
+    max_sub = X - max_keepdims
+    exp_arr = np.exp(max_sub)
+    sum_keepdims = np.reshape(np.sum(exp_arr, axis=axis), reduced_shape)
+    log_sum = np.log(sum_keepdims)
+    return max_sub - log_sum
+
+
+def sum_(*inputs):
+    """PureSum: all inputs have the output's shape, added left to right (pure_implementations.py:529-591)."""
+    out = inputs[0]
+    for x in inputs[1:]:
+        out = out + x
+    return out
+
+
 def layer_normalization(X, gamma, beta=None, axis=-1, epsilon=1e-5):
     """LayerNormalization as the nine-node chain the reference actually runs
     (there is no LayerNormalization node at opset 12): ReduceMean, Sub, Pow(2),
@@ -240,6 +276,51 @@ def div(A, B):
 
 def sqrt(X):
     return np.sqrt(X)
+
+
+def log(X):
+    """PureLog (pure_implementations.py:23-38)."""
+    return np.log(X)
+
+
+def tanh(X):
+    """Tanh via python_pure_op_implementation (pure_implementations.py:296-298)."""
+    return np.tanh(X)
+
+
+def reciprocal(X):
+    """PureReciprocal: dtype(1) / x (pure_implementations.py:275-293)."""
+    return (np.asarray(1, dtype=X.dtype) / X).astype(X.dtype, copy=False)
+
+
+def softplus(X):
+    """Softplus exactly as written in the reference, log(1 + exp(x)), in the input dtype
+    (pure_implementations.py:696-698): overflows to inf where exp does."""
+    with np.errstate(over="ignore"):
+        return np.log(np.asarray(1, dtype=X.dtype) + np.exp(X)).astype(X.dtype, copy=False)
+
+
+def sigmoid(X):
+    """PureSigmoid: dtype(1) / (dtype(1) + exp(-x)) (pure_implementations.py:701-712)."""
+    one = np.asarray(1, dtype=X.dtype)
+    with np.errstate(over="ignore"):
+        return (one / (one + np.exp(-X))).astype(X.dtype, copy=False)
+
+
+def exp(X):
+    """ONNX Exp (no pure expansion in the reference; ONNX Runtime runs it there)."""
+    with np.errstate(over="ignore"):
+        return np.exp(X)
+
+
+def neg(X):
+    """ONNX Neg (no pure expansion in the reference)."""
+    return np.negative(X)
+
+
+def abs(X):  # noqa: A001 (named after the ONNX op)
+    """ONNX Abs (no pure expansion in the reference)."""
+    return np.abs(X)
 
 
 def pow(X, Y):  # noqa: A001 (named after the ONNX op)

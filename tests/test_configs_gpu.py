@@ -362,3 +362,42 @@ def test_pad_then_conv_matches_padding_by_hand():
     xp = np.pad(x, ((0, 0), (0, 0), (1, 3), (2, 0)))
     assert rel_err(O.conv2d(xp, w, None, pads=(1, 0, 0, 2)), got) < FP32_REL_TOL
     assert model.compile_and_init().num_launches == 1
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_tanh_gelu_silu_softplus_chain_values(fuse):
+    from test_fusion import _chain_model, _tanh_gelu_and_silu_nodes
+    nodes, consts = _tanh_gelu_and_silu_nodes()
+    x = np.random.default_rng(8).normal(scale=2, size=(4, 8)).astype(np.float32)
+    got = donnx.ONNXModel(f"tanh_chain_{fuse}", _chain_model(nodes, consts), fuse=fuse)(x)
+    x64 = x.astype(np.float64)
+    gelu = 0.5 * x64 * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x64 + 0.044715 * x64 ** 3)))
+    silu = gelu / (1.0 + np.exp(-gelu))
+    assert np.allclose(got, np.log1p(np.exp(silu)), rtol=1e-5, atol=1e-6)
+
+
+def test_classifier_head_with_log_softmax_reductions_and_sum():
+    """Gemm -> LogSoftmax, plus ReduceSum / ReduceMax / ReduceMin of the logits and a three-input Sum, in one
+    ONNXModel: the operators of pure_implementations.py:301-343, 529-616 on the importer's path."""
+    H, T = proto.helper, proto.TensorProto
+    rng = np.random.default_rng(9)
+    x = rng.normal(size=(16, 64)).astype(np.float32)
+    w = rng.normal(scale=0.2, size=(10, 64)).astype(np.float32)
+    b = rng.normal(scale=0.1, size=(10, )).astype(np.float32)
+    nodes = [H.make_node("Gemm", ["x", "w", "b"], ["logits"], transB=1),
+             H.make_node("LogSoftmax", ["logits"], ["logp"], axis=1),
+             H.make_node("ReduceSum", ["logits"], ["rs"], axes=[1], keepdims=1),
+             H.make_node("ReduceMax", ["logits"], ["rmax"], axes=[1], keepdims=1),
+             H.make_node("ReduceMin", ["logits"], ["rmin"], axes=[0], keepdims=0),
+             H.make_node("Sum", ["logp", "logits", "logp"], ["total"])]
+    outs = [("logp", [16, 10]), ("rs", [16, 1]), ("rmax", [16, 1]), ("rmin", [10]), ("total", [16, 10])]
+    g = H.make_graph(nodes, "head", [H.make_tensor_value_info("x", T.FLOAT, [16, 64])],
+                     [H.make_tensor_value_info(n, T.FLOAT, s) for n, s in outs],
+                     initializer=[proto.numpy_helper.from_array(w, "w"), proto.numpy_helper.from_array(b, "b")])
+    model = donnx.ONNXModel("classifier_head", H.make_model(g, opset_imports=[H.make_opsetid("", 12)]))
+    logp, rs, rmax, rmin, total = model(x)
+    logits = O.gemm(x, w, b, transB=1)
+    assert rel_err(O.log_softmax(logits, axis=1), logp) < FP32_REL_TOL
+    assert rel_err(O.reduce_sum(logits, [1]), rs) < FP32_REL_TOL
+    assert np.allclose(rmax, O.reduce_max(logits, [1]), rtol=1e-5) and np.allclose(rmin, O.reduce_min(logits, [0], 0), rtol=1e-5)
+    assert rel_err(O.sum_(O.log_softmax(logits, axis=1), logits, O.log_softmax(logits, axis=1)), total) < FP32_REL_TOL

@@ -294,6 +294,39 @@ def test_unary_ops(shape):
     assert rel_err(O.sqrt(np.abs(X)), Y) < 1e-6
 
 
+@pytest.mark.parametrize("shape", [(8, 16, 3072), (7, ), (1, 3, 5), (4097, )])
+@pytest.mark.parametrize("op, conns, positive", [("Log", ("input", "output"), True), ("Tanh", ("input", "output"), False),
+                                                 ("Exp", ("input", "output"), False), ("Sigmoid", ("X", "Y"), False),
+                                                 ("Softplus", ("X", "Y"), False), ("Reciprocal", ("X", "Y"), True),
+                                                 ("Neg", ("X", "Y"), False), ("Abs", ("X", "Y"), False)])
+def test_more_unary_ops(op, conns, positive, shape):
+    """The unary maps of pure_implementations.py:23-38, 275-298, 696-712 (and Exp, Neg, Abs): every element
+    within a few fp32 roundings of the oracle's value."""
+    X = np.random.default_rng(31).normal(scale=3, size=shape).astype(np.float32)
+    if positive:
+        X = np.abs(X) + np.float32(0.05)
+    Y = np.zeros_like(X)
+    getattr(donnx, "ONNX" + op)(**{conns[0]: X, conns[1]: Y})
+    expected = getattr(O, op.lower())(X)
+    if op in ("Neg", "Abs"):
+        assert np.array_equal(expected, Y)
+    else:
+        assert np.allclose(Y, expected, rtol=2e-6, atol=2e-7), np.abs(Y - expected).max()
+
+
+def test_softplus_sigmoid_extremes():
+    """Same behaviour as the reference's formulas at the ends: log(1 + exp(x)) overflows where exp does and
+    is exactly 0 far to the left; the sigmoid saturates at 0 and 1 without NaN."""
+    X = np.array([-200.0, -104.0, -20.0, 0.0, 20.0, 88.0, 89.0, 200.0], dtype=np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXSoftplus(X=X, Y=Y)
+    expected = O.softplus(X)
+    assert np.array_equal(np.isinf(expected), np.isinf(Y)) and np.allclose(Y[:-2], expected[:-2], rtol=2e-6, atol=1e-7)
+    donnx.ONNXSigmoid(X=X, Y=Y)
+    assert not np.isnan(Y).any() and Y[0] == 0.0 and Y[-1] == 1.0 and Y[3] == 0.5
+    assert np.allclose(Y, O.sigmoid(X), rtol=2e-6, atol=1e-30)
+
+
 @pytest.mark.parametrize("shape, axes, keepdims", [((8, 16, 768), [-1], 1), ((5, 33), [1], 0), ((4, 6, 10), [1], 1),
                                                    ((3, 4, 5, 6), [1, 2], 0), ((7, 9), [0, 1], 1), ((2, 4100), [-1], 1)])
 def test_reduce_mean(shape, axes, keepdims):
@@ -302,6 +335,68 @@ def test_reduce_mean(shape, axes, keepdims):
     Y = np.zeros(expected.shape, np.float32)
     donnx.ONNXReduceMean(data=X, reduced=Y, axes=axes, keepdims=keepdims)
     assert rel_err(expected, Y) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("shape, axes, keepdims", [((8, 16, 768), [-1], 1), ((5, 33), [1], 0), ((4, 6, 10), [1], 1),
+                                                   ((3, 4, 5, 6), [1, 2], 0), ((7, 9), [0, 1], 1), ((2, 4100), [-1], 1),
+                                                   ((4100, 3), [0], 0)])
+@pytest.mark.parametrize("op", ["ReduceSum", "ReduceMax", "ReduceMin"])
+def test_reduce_sum_max_min(op, shape, axes, keepdims):
+    """np.sum / np.max / np.min over ``axes`` (pure_implementations.py:301-343): extrema exact, sums against
+    the double-precision sum."""
+    X = np.random.default_rng(17).normal(1.0, 2.0, size=shape).astype(np.float32)
+    oracle = {"ReduceSum": O.reduce_sum, "ReduceMax": O.reduce_max, "ReduceMin": O.reduce_min}[op]
+    expected = oracle(X.astype(np.float64), axes, keepdims)
+    Y = np.zeros(expected.shape, np.float32)
+    getattr(donnx, "ONNX" + op)(data=X, reduced=Y, axes=axes, keepdims=keepdims)
+    if op == "ReduceSum":
+        assert rel_err(expected, Y) < FP32_REL_TOL
+        abs_sum = O.reduce_sum(np.abs(X).astype(np.float64), axes, keepdims)   # every element, not only the norm
+        assert (np.abs(Y - expected) <= 5e-6 * abs_sum).all()
+    else:
+        assert np.array_equal(expected.astype(np.float32), Y)
+
+
+def test_reduce_max_min_propagate_nan():
+    X = np.random.default_rng(18).normal(size=(6, 50)).astype(np.float32)
+    X[2, 17] = np.nan
+    for op, oracle in (("ReduceMax", O.reduce_max), ("ReduceMin", O.reduce_min)):
+        for axes in ([1], [0]):
+            expected = oracle(X, axes, 0)
+            Y = np.zeros(expected.shape, np.float32)
+            getattr(donnx, "ONNX" + op)(data=X, reduced=Y, axes=axes, keepdims=0)
+            assert np.array_equal(expected, Y, equal_nan=True), (op, axes)
+
+
+@pytest.mark.parametrize("shape, axis", [((8, 12, 128, 128), -1), ((5, 48), -1), ((3, 1000), 1), ((2, 5000), -1),
+                                         ((3, 30), -1), ((3, 17, 5, 9), 1), ((4, 6, 48), 0), ((3, 1), -1)])
+def test_log_softmax(shape, axis):
+    """PureLogSoftmax (pure_implementations.py:594-616); also exp(result) must sum to one along the axis."""
+    X = np.random.default_rng(19).normal(scale=4, size=shape).astype(np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXLogSoftmax(input=X, output=Y, axis=axis)
+    expected = O.log_softmax(X.astype(np.float64), axis=axis)
+    assert np.allclose(Y, expected, rtol=1e-5, atol=2e-6), np.abs(Y - expected).max()
+    assert np.allclose(np.exp(Y.astype(np.float64)).sum(axis), 1.0, atol=1e-4)
+    assert np.allclose(Y, torch.nn.functional.log_softmax(torch.from_numpy(X), dim=axis).numpy(), rtol=1e-5, atol=2e-6)
+
+
+def test_log_softmax_large_values():
+    X = np.array([[1000.0, 999.0, -1000.0, 0.0]] * 3, np.float32)
+    Y = np.zeros_like(X)
+    donnx.ONNXLogSoftmax(input=X, output=Y, axis=1)
+    assert np.isfinite(Y).all() and np.allclose(Y, O.log_softmax(X.astype(np.float64), axis=1), rtol=1e-6)
+
+
+@pytest.mark.parametrize("count", [1, 2, 3, 4])
+@pytest.mark.parametrize("shape", [(8, 16, 768), (7, ), (3, 5)])
+def test_sum(count, shape):
+    """PureSum (pure_implementations.py:529-591): inputs of one shape, added left to right -- bit-exact."""
+    rng = np.random.default_rng(20)
+    xs = [rng.normal(size=shape).astype(np.float32) for _ in range(count)]
+    Y = np.zeros(shape, np.float32)
+    donnx.ONNXSum(**{f"data_0__{i}": x for i, x in enumerate(xs)}, sum=Y)
+    assert np.array_equal(O.sum_(*xs), Y)
 
 
 def test_pow():

@@ -142,13 +142,62 @@ def test_gelu_pattern_variants():
     bad = dict(consts, r2=1.5)
     calls = _launches(donnx.ONNXModel("g", _chain_model(variants["div, (x * t) * 0.5"], bad)))
     assert [f for f, _ in calls] == ["mi355x_eltwise_program_f32"] and calls[0][1][8] == 5
-    # erf(x / sqrt 2) with another reader of the intermediate is not Gelu either: two programs, split at the
-    # value that has two readers
+    # erf(x / sqrt 2) with another reader of the intermediate is not Gelu either; both readers are elementwise,
+    # so the value stays in a register of one five-instruction program
     nodes = variants["div, (x * t) * 0.5"][:-1] + [mk("Mul", ["u", "e"], ["y"])]
     calls = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))
-    assert sorted((f, a[8]) for f, a in calls) == [("mi355x_eltwise_program_f32", 2), ("mi355x_eltwise_program_f32", 3)]
+    assert [(f, a[8]) for f, a in calls] == [("mi355x_eltwise_program_f32", 5)]
     unfused = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts), fuse=False))
     assert len(unfused) == 5
+
+
+def _tanh_gelu_and_silu_nodes():
+    """x -> tanh-approximated Gelu (eight elementwise nodes) -> SiLU (x * sigmoid(x)) -> Softplus."""
+    mk = H.make_node
+    consts = {"c": 0.044715, "k": (2.0 / np.pi) ** 0.5, "one": 1.0, "half": 0.5, "three": 3.0}
+    nodes = [mk("Pow", ["x", "three"], ["x3"]), mk("Mul", ["x3", "c"], ["cx3"]), mk("Add", ["x", "cx3"], ["inner"]),
+             mk("Mul", ["inner", "k"], ["scaled"]), mk("Tanh", ["scaled"], ["t"]), mk("Add", ["t", "one"], ["t1"]),
+             mk("Mul", ["x", "t1"], ["xt"]), mk("Mul", ["xt", "half"], ["gelu"]),
+             mk("Sigmoid", ["gelu"], ["sg"]), mk("Mul", ["gelu", "sg"], ["silu"]), mk("Softplus", ["silu"], ["y"])]
+    return nodes, consts
+
+
+def test_tanh_sigmoid_softplus_chains_become_one_program():
+    # the unary maps of pure_implementations.py:275-298, 696-712 join elementwise groups like Relu / Erf / Sqrt do
+    nodes, consts = _tanh_gelu_and_silu_nodes()
+    calls = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts)))
+    assert [f for f, _ in calls] == ["mi355x_eltwise_program_f32"] and calls[0][1][8] == 11
+    assert calls[0][1][1] == 1 and calls[0][1][3] == 0           # one tensor read, no vectors
+    unfused = _launches(donnx.ONNXModel("g", _chain_model(nodes, consts), fuse=False))
+    assert [f for f, _ in unfused] == ["mi355x_eltwise_f32"] * 11
+    assert sorted(a[0] for _, a in unfused) == sorted([4, 2, 0, 2, 22, 0, 2, 2, 23, 2, 24])
+
+
+def test_elementwise_groups_respect_the_kernel_limits_and_outside_readers():
+    mk = H.make_node
+    # 20 dependent nodes: more than one program holds (16 instructions) -> two programs, 20 instructions in all
+    nodes = [mk("Tanh" if i % 2 else "Abs", ["x" if i == 0 else f"v{i - 1}"], [f"v{i}" if i < 19 else "y"]) for i in range(20)]
+    calls = _launches(donnx.ONNXModel("g", _chain_model(nodes, {})))
+    assert [f for f, _ in calls] == ["mi355x_eltwise_program_f32"] * 2 and sum(a[8] for _, a in calls) == 20
+    assert max(a[8] for _, a in calls) <= 16
+    # nine values alive at once do not fit eight registers: the group shrinks until it does
+    nodes = [mk("Tanh" if i % 2 else "Abs", ["x"], [f"b{i}"]) for i in range(9)]
+    nodes += [mk("Sigmoid", [f"b{i}"], [f"c{i}"]) for i in range(9)]
+    acc = "c0"
+    for i in range(1, 9):
+        nodes.append(mk("Mul", [acc, f"c{i}"], [f"m{i}" if i < 8 else "y"]))
+        acc = f"m{i}"
+    model = donnx.ONNXModel("g", _chain_model(nodes, {}))
+    calls = _launches(model)
+    assert sum(a[8] if f == "mi355x_eltwise_program_f32" else 1 for f, a in calls) == 26 and len(calls) <= 4
+    for f, a in calls:
+        assert f == "mi355x_eltwise_f32" or (a[8] <= 16 and max((w >> 8) & 255 for w in a[7].values) < 8)
+    # an intermediate that something outside the group reads (here: a MatMul) is materialised, not absorbed
+    nodes = [mk("Tanh", ["x"], ["t"]), mk("Sigmoid", ["t"], ["s"]), mk("Mul", ["t", "s"], ["p"]),
+             mk("MatMul", ["t", "w"], ["q"]), mk("Add", ["p", "q"], ["y"])]
+    g = _chain_model(nodes, {"w": np.eye(8)})
+    calls = _launches(donnx.ONNXModel("g", g))
+    assert sorted(f for f, _ in calls) == ["mi355x_eltwise_f32", "mi355x_eltwise_program_f32", "mi355x_gemm_f32"]
 
 
 def test_layernorm_pattern_needs_the_exact_chain():

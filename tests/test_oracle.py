@@ -194,6 +194,52 @@ def test_gelu_erf_relu_closed_forms():
     assert O.relu(x).dtype == np.float32
 
 
+def test_unary_maps_closed_forms():
+    """Log, Tanh, Reciprocal, Softplus, Sigmoid (and Exp, Neg, Abs) against the math module in double, value
+    by value, plus what fixes the formula: the reference's Softplus is log(1 + exp(x)) literally, so it
+    overflows at x = 89 and is exactly 0 where exp(x) is below half an ulp of 1."""
+    rng = np.random.default_rng(21)
+    x = rng.normal(scale=3, size=500).astype(np.float32)
+    x64 = x.astype(np.float64)
+    each = lambda f, v: np.array([f(t) for t in v])
+    assert np.allclose(O.tanh(x), each(math.tanh, x64), rtol=3e-7, atol=1e-7)
+    assert np.allclose(O.log(np.abs(x) + 0.1), each(math.log, np.abs(x).astype(np.float32).astype(np.float64) + np.float32(0.1)),
+                       rtol=1e-6, atol=2e-7)
+    assert np.allclose(O.reciprocal(x), 1.0 / x64, rtol=2e-7)
+    assert np.allclose(O.softplus(x), each(lambda t: math.log1p(math.exp(t)), x64), rtol=1e-6, atol=1e-7)
+    assert np.allclose(O.sigmoid(x), each(lambda t: 1.0 / (1.0 + math.exp(-t)), x64), rtol=3e-7)
+    assert np.allclose(O.sigmoid(x) + O.sigmoid(-x), 1.0, atol=2e-7)        # symmetry
+    assert np.allclose(O.exp(x), each(math.exp, x64), rtol=3e-7)
+    assert np.array_equal(O.neg(x), -x) and np.array_equal(O.abs(x), np.abs(x))
+    assert O.tanh(x).dtype == O.softplus(x).dtype == O.sigmoid(x).dtype == O.reciprocal(x).dtype == np.float32
+    edge = np.array([89.0, -20.0, 0.0], dtype=np.float32)
+    sp = O.softplus(edge)
+    assert np.isinf(sp[0]) and sp[1] == 0.0 and sp[2] == np.float32(math.log(2.0))
+    assert O.sigmoid(np.array([-100.0, 100.0], np.float32)).tolist() == [0.0, 1.0]
+
+
+def test_reductions_log_softmax_sum_closed_forms():
+    """ReduceSum / Max / Min against explicit loops, LogSoftmax against log(softmax) in double and its
+    normalisation, Sum against left-to-right addition."""
+    rng = np.random.default_rng(22)
+    x = rng.normal(size=(3, 5, 7)).astype(np.float32)
+    s = O.reduce_sum(x, [1], keepdims=0)
+    assert s.shape == (3, 7) and s.dtype == np.float32
+    for i in range(3):
+        for k in range(7):
+            col = [float(x[i, j, k]) for j in range(5)]
+            assert abs(s[i, k] - math.fsum(col)) < 1e-5
+            assert O.reduce_max(x, [1], 0)[i, k] == max(col) and O.reduce_min(x, [1], 0)[i, k] == min(col)
+    assert O.reduce_max(x, [0, 2]).shape == (1, 5, 1) and O.reduce_sum(x, [0, 1, 2], keepdims=0).shape == ()
+    ls = O.log_softmax(x, axis=1)
+    assert np.allclose(ls, np.log(O.softmax(x.astype(np.float64), axis=1)), atol=1e-6)
+    assert np.allclose(np.exp(ls.astype(np.float64)).sum(1), 1.0, atol=1e-6)
+    assert np.allclose(O.log_softmax(x + 100.0, axis=1), ls, atol=1e-4)        # shift invariance
+    assert np.allclose(O.log_softmax(np.zeros((2, 8), np.float32)), -math.log(8.0))
+    a, b, c = (rng.normal(size=(4, 4)).astype(np.float32) for _ in range(3))
+    assert np.array_equal(O.sum_(a, b, c), (a + b) + c) and np.array_equal(O.sum_(a), a)
+
+
 def test_pow_and_reduce_mean_closed_forms():
     rng = np.random.default_rng(21)
     x = rng.normal(size=(3, 5, 7)).astype(np.float32)

@@ -4,7 +4,8 @@ evaluation of the same node list must agree.
 The fusion pass rewrites chains (bias / scale / activation / residual into GEMM epilogues, Reshape and
 Transpose into operand strides, shared-input MatMuls into one, attention into one node); what it must
 never do is change the value. Each seeded graph is a random walk over MatMul (constant weight, optional
-bias as either Add operand), Gemm, scalar Mul / Div before or after a product, Relu / Gelu, residual Adds
+bias as either Add operand), Gemm, scalar Mul / Div before or after a product, Relu / Gelu / Tanh / Sigmoid /
+Softplus / Abs / Neg, residual Adds
 with earlier values, LayerNormalization, Softmax, head split / merge (Reshape + Transpose) and
 activation-by-activation MatMuls, with values that have several readers now and then. Without a GPU the
 graphs are imported, fused and expanded (structure only); with one, all three results are compared."""
@@ -70,7 +71,7 @@ def random_graph(seed):
         if kind == "linear":
             cur = linear(cur, int(rng.choice([32, 64, 96, 128])))
         elif kind == "act":
-            cur = g.node(str(rng.choice(["Relu", "Gelu"])), [cur], shape)
+            cur = g.node(str(rng.choice(["Relu", "Gelu", "Tanh", "Sigmoid", "Softplus", "Abs", "Neg"])), [cur], shape)
         elif kind == "scale":
             c = g.const(np.float32(rng.choice([0.5, 2.0, 0.125, -1.5])), "s")
             op = str(rng.choice(["Mul", "Div"]))
@@ -140,7 +141,7 @@ def evaluate_with_oracle(model, x):
             y = O.gemm(i[0], i[1], i[2] if len(i) > 2 else None, transB=int(a.get("transB", 0)))
         elif op in ("Add", "Mul", "Div"):
             y = getattr(O, op.lower())(i[0], i[1])
-        elif op in ("Relu", "Gelu"):
+        elif op in ("Relu", "Gelu", "Tanh", "Sigmoid", "Softplus", "Abs", "Neg"):
             y = getattr(O, op.lower())(i[0])
         elif op == "LayerNormalization":
             y = O.layer_normalization(i[0], i[1], i[2], axis=-1, epsilon=float(a["epsilon"]))
