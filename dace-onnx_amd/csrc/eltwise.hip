@@ -139,6 +139,16 @@ __global__ __launch_bounds__(256) void permute_tiled(const uint32_t* __restrict_
     }
 }
 
+// ONNX Cast: Y[i] = (TO)X[i]; to bool is X[i] != 0 (stored as one byte).
+template <class FROM, class TO, bool TO_BOOL>
+__global__ __launch_bounds__(256) void cast_kernel(const FROM* __restrict__ X, TO* __restrict__ Y, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        if constexpr (TO_BOOL) Y[i] = (TO)(X[i] != (FROM)0);
+        else Y[i] = (TO)X[i];
+    }
+}
+
 // Merge adjacent dims (d, d+1) when both operands step through them as one.
 static void collapse(IndexMap& m, bool use_b) {
     // drop size-1 dims
@@ -245,6 +255,45 @@ extern "C" int mi355x_eltwise_f32(int op, const float* A, const float* B, float*
         case MI355X_OP_NEG: return launch_eltwise<MI355X_OP_NEG>(A, B, C, m, st);
         case MI355X_OP_ABS: return launch_eltwise<MI355X_OP_ABS>(A, B, C, m, st);
         default: return set_error(MI355X_ERR_INVALID_ARGUMENT, "eltwise: unknown op %d", op);
+    }
+}
+
+namespace mi355x {
+
+template <class FROM>
+static int launch_cast_from(const void* X, void* Y, int to_type, int64_t n, hipStream_t st) {
+    const FROM* x = static_cast<const FROM*>(X);
+    const dim3 grid(grid_for(n)), block(256);
+    switch (to_type) {
+        case MI355X_TYPE_FLOAT: hipLaunchKernelGGL((cast_kernel<FROM, float, false>), grid, block, 0, st, x, static_cast<float*>(Y), n); break;
+        case MI355X_TYPE_DOUBLE: hipLaunchKernelGGL((cast_kernel<FROM, double, false>), grid, block, 0, st, x, static_cast<double*>(Y), n); break;
+        case MI355X_TYPE_INT32: hipLaunchKernelGGL((cast_kernel<FROM, int32_t, false>), grid, block, 0, st, x, static_cast<int32_t*>(Y), n); break;
+        case MI355X_TYPE_INT64: hipLaunchKernelGGL((cast_kernel<FROM, int64_t, false>), grid, block, 0, st, x, static_cast<int64_t*>(Y), n); break;
+        case MI355X_TYPE_INT8: hipLaunchKernelGGL((cast_kernel<FROM, int8_t, false>), grid, block, 0, st, x, static_cast<int8_t*>(Y), n); break;
+        case MI355X_TYPE_UINT8: hipLaunchKernelGGL((cast_kernel<FROM, uint8_t, false>), grid, block, 0, st, x, static_cast<uint8_t*>(Y), n); break;
+        case MI355X_TYPE_BOOL: hipLaunchKernelGGL((cast_kernel<FROM, uint8_t, true>), grid, block, 0, st, x, static_cast<uint8_t*>(Y), n); break;
+        default: return set_error(MI355X_ERR_INVALID_ARGUMENT, "cast: unsupported target type %d", to_type);
+    }
+    return check_launch("cast");
+}
+
+}  // namespace mi355x
+
+extern "C" int mi355x_cast(const void* X, int from_type, void* Y, int to_type, int64_t n, void* stream) {
+    using namespace mi355x;
+    MI355X_REQUIRE(n >= 0, "cast: negative element count %lld", (long long)n);
+    if (n == 0) return MI355X_OK;
+    MI355X_REQUIRE(X && Y, "cast: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (from_type) {
+        case MI355X_TYPE_FLOAT: return launch_cast_from<float>(X, Y, to_type, n, st);
+        case MI355X_TYPE_DOUBLE: return launch_cast_from<double>(X, Y, to_type, n, st);
+        case MI355X_TYPE_INT32: return launch_cast_from<int32_t>(X, Y, to_type, n, st);
+        case MI355X_TYPE_INT64: return launch_cast_from<int64_t>(X, Y, to_type, n, st);
+        case MI355X_TYPE_INT8: return launch_cast_from<int8_t>(X, Y, to_type, n, st);
+        case MI355X_TYPE_UINT8:
+        case MI355X_TYPE_BOOL: return launch_cast_from<uint8_t>(X, Y, to_type, n, st);
+        default: return set_error(MI355X_ERR_INVALID_ARGUMENT, "cast: unsupported source type %d", from_type);
     }
 }
 

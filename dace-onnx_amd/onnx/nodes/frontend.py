@@ -35,8 +35,13 @@ def call_onnx_op(cls, **kwargs):
     cls.__init__(node, "ONNX" + schema.name, **attrs)
     state.add_node(node)
     call_args = {}
+    # small host integer arrays (Slice's starts / ends / axes / steps, a Reshape target) are compile-time
+    # constants of this one-node graph, as initializers are in an imported model
+    sdfg._constant_inputs = {}
     for conn, value in list(inputs.items()) + list(outputs.items()):
         arr = "__" + conn
+        if conn in inputs and isinstance(value, np.ndarray) and np.issubdtype(value.dtype, np.integer) and value.size <= 64:
+            sdfg._constant_inputs[arr] = value.copy()
         shape = tuple(value.shape) if hasattr(value, "shape") else ()
         dtype = value.dtype if hasattr(value, "dtype") else np.asarray(value).dtype
         sdfg.add_array(arr, shape, dace.typeclass_of(dtype))

@@ -680,6 +680,80 @@ class MI355XTranspose(ONNXForward):
             I64Array([X.strides[p] for p in perm]), Stream()])
 
 
+# ONNX TensorProto data types the cast kernel converts between (the values of Cast's ``to``)
+_CAST_TYPES = {"float32": 1, "uint8": 2, "int8": 3, "int32": 6, "int64": 7, "bool_": 9, "float64": 11}
+
+
+@op_implementation(op="Cast", name=IMPLEMENTATION_NAME)
+class MI355XCast(ONNXForward):
+    """Elementwise conversion in one pass (PureCast, :382-430: a map of ``__output = __input``)."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "input")
+        Y = out_desc_with_name(node, state, sdfg, "output")
+        return X.dtype.name in _CAST_TYPES and Y.dtype.name in _CAST_TYPES and _contig(X, Y) and \
+            tuple(X.shape) == tuple(Y.shape) and (node.to is None or int(node.to) == _CAST_TYPES[Y.dtype.name])
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "input")
+        Y = out_desc_with_name(node, state, sdfg, "output")
+        return kernel_call_for_node(node, state, "mi355x_cast", [
+            Ptr("input"), _CAST_TYPES[X.dtype.name], Ptr("output"), _CAST_TYPES[Y.dtype.name], int(X.total_size), Stream()])
+
+
+@op_implementation(op="Slice", name=IMPLEMENTATION_NAME)
+class MI355XSlice(ONNXForward):
+    """Slice with constant ``starts`` / ``ends`` / ``axes`` / ``steps`` as one strided gather of 4-byte
+    elements: any axes, any non-zero steps. PureSlice (:619-693) covers axis 0 with step 1 and explicit
+    ``axes`` and ``steps`` only and leaves the rest to ONNX Runtime."""
+
+    @staticmethod
+    def _ranges(node, state, sdfg):
+        """slice_ranges(...) of the node, or None when an index input is not a constant."""
+        from ...onnx.shape_inference import slice_ranges, ShapeInferenceError
+        model = getattr(sdfg, "_parent_onnx_model", None)
+        idx = []
+        for name in ("starts", "ends", "axes", "steps"):
+            if not _has_input(node, state, name):
+                idx.append(None)
+                continue
+            edge = [e for e in state.in_edges(node) if e.dst_conn == name][0]
+            if state.in_edges(edge.src):
+                return None             # computed by another node
+            if model is not None and edge.src.data in model.clean_weights:
+                idx.append([int(v) for v in model.clean_weights[edge.src.data].detach().cpu().reshape(-1).tolist()])
+            elif edge.src.data in getattr(sdfg, "_constant_inputs", {}):       # the call form donnx.ONNXSlice(...)
+                idx.append([int(v) for v in sdfg._constant_inputs[edge.src.data].reshape(-1)])
+            else:
+                return None
+        if idx[0] is None or idx[1] is None:
+            return None
+        try:
+            return slice_ranges(in_desc_with_name(node, state, sdfg, "data").shape, *idx)
+        except ShapeInferenceError:
+            return None
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "data")
+        Y = out_desc_with_name(node, state, sdfg, "output")
+        if X.dtype != Y.dtype or X.dtype.bytes != 4 or not _contig(X, Y) or not 1 <= len(X.shape) <= MAX_ELTWISE_DIMS:
+            return False
+        ranges = MI355XSlice._ranges(node, state, sdfg)
+        return ranges is not None and tuple(Y.shape) == tuple(c for _, _, c in ranges)
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "data")
+        ranges = MI355XSlice._ranges(node, state, sdfg)
+        offset = sum(first * stride for (first, _, count), stride in zip(ranges, X.strides)) if all(c for _, _, c in ranges) else 0
+        return kernel_call_for_node(node, state, "mi355x_permute_b32", [
+            Ptr("data", offset), Ptr("output"), len(ranges), I64Array([c for _, _, c in ranges]),
+            I64Array([stride * step for (_, step, _), stride in zip(ranges, X.strides)]), Stream()])
+
+
 def _alias_impl(op_name, in_conn, out_conn):
     @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
     class Impl(ONNXForward):

@@ -162,6 +162,15 @@ SCHEMAS: typing.List[ONNXSchema] = [
 ] + [
     _unary("LogSoftmax", 11, "input", "output", attributes=[ONNXAttribute("axis", _A.Int, 1)],
            doc="Log of the softmax along `axis`."),
+    ONNXSchema("Cast", 9, [ONNXParameter("input", "T1")], [ONNXParameter("output", "T2")],
+               [ONNXAttribute("to", _A.Int, required=True)],
+               [ONNXTypeConstraint("T1", _ANY), ONNXTypeConstraint("T2", _ANY)], "Elementwise conversion to the type `to`."),
+    ONNXSchema("Slice", 11,
+               [ONNXParameter("data", "T"), ONNXParameter("starts", "Tind"), ONNXParameter("ends", "Tind"),
+                ONNXParameter("axes", "Tind", _O), ONNXParameter("steps", "Tind", _O)],
+               [ONNXParameter("output", "T")], (),
+               [ONNXTypeConstraint("T", _ANY), ONNXTypeConstraint("Tind", [dace.int32, dace.int64])],
+               "data[starts:ends:steps] along `axes` (numpy slicing semantics, bounds clamped)."),
     ONNXSchema("Sum", 8, [ONNXParameter("data_0", "T", ONNXParameterType.Variadic)], [ONNXParameter("sum", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS)], "Elementwise sum of the inputs."),
 ]

@@ -26,6 +26,25 @@ def _conv_out(size, k, stride, dil, pad_lo, pad_hi):
     return (size + pad_lo + pad_hi - ((k - 1) * dil + 1)) // stride + 1
 
 
+def slice_ranges(shape, starts, ends, axes=None, steps=None):
+    """Per axis of ``shape``: (first index, step, number of elements) of an ONNX Slice, with the operator's
+    clamping rules (negative indices count from the end, out-of-range bounds are clamped -- which is what
+    Python slicing does; ``ends`` of INT64_MAX is the exporters' "to the end")."""
+    rank = len(shape)
+    starts, ends = [int(v) for v in starts], [int(v) for v in ends]
+    axes = [int(v) for v in axes] if axes is not None else list(range(len(starts)))
+    steps = [int(v) for v in steps] if steps is not None else [1] * len(starts)
+    if not len(starts) == len(ends) == len(axes) == len(steps):
+        raise ShapeInferenceError("Slice: starts, ends, axes and steps differ in length")
+    out = [(0, 1, int(d)) for d in shape]
+    for s, e, ax, st in zip(starts, ends, axes, steps):
+        if not -rank <= ax < rank or st == 0:
+            raise ShapeInferenceError(f"Slice: axis {ax} outside rank {rank}, or a zero step")
+        selected = range(*slice(s, e, st).indices(int(shape[ax % rank])))
+        out[ax % rank] = (selected.start, st, len(selected))
+    return out
+
+
 def _infer_node(node, shapes, types, constants):
     """Return [(shape, elem_type)] for each output of ``node``."""
     a = _attrs(node)
@@ -76,7 +95,14 @@ def _infer_node(node, shapes, types, constants):
         return [(tuple(ins[0][p] for p in perm), tys[0])]
     if op == "Reshape":
         if node.input[1] not in constants:
-            raise ShapeInferenceError(f"Reshape '{node.name}': the shape input must be a constant initializer")
+            # the shape is computed by other nodes (left in the graph when constants are not folded): the model
+            # must then declare the result's shape, which is all the expansion needs (PureReshape reads the
+            # output descriptor too, pure_implementations.py:497)
+            declared = shapes.get(node.output[0])
+            if declared is None or int(np.prod(declared)) != (int(np.prod(ins[0])) if len(ins[0]) else 1):
+                raise ShapeInferenceError(f"Reshape '{node.name}': the shape input is not a constant initializer and "
+                                          "the model declares no (matching) shape for the result")
+            return [(tuple(declared), tys[0])]
         target = [int(v) for v in constants[node.input[1]].ravel()]
         total = int(np.prod(ins[0])) if len(ins[0]) else 1
         out = [ins[0][i] if v == 0 else v for i, v in enumerate(target)]
@@ -99,6 +125,16 @@ def _infer_node(node, shapes, types, constants):
     if op == "Flatten":
         axis = a.get("axis", 1) % (len(ins[0]) + 1) if a.get("axis", 1) < 0 else a.get("axis", 1)
         return [((int(np.prod(ins[0][:axis])) if axis else 1, int(np.prod(ins[0][axis:]))), tys[0])]
+    if op == "Cast":
+        return [(ins[0], int(a["to"]))]
+    if op == "Slice":
+        idx = []
+        for k in range(1, 5):
+            name = node.input[k] if len(node.input) > k else ""
+            if name and name not in constants:
+                raise ShapeInferenceError(f"Slice '{node.name}': input '{name}' must be a constant initializer")
+            idx.append([int(v) for v in constants[name].ravel()] if name else None)
+        return [(tuple(c for _, _, c in slice_ranges(ins[0], *idx)), tys[0])]
     if op == "Sum":
         return [(tuple(np.broadcast_shapes(*ins)), tys[0])]
     if op in ("ReduceMean", "ReduceSum", "ReduceMax", "ReduceMin"):

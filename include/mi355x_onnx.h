@@ -248,9 +248,28 @@ int mi355x_eltwise_program_f32(const float* const* tensors, int n_tensors,
 
 /* ONNX Transpose (and any strided gather), 4-byte elements:
  *   Y (C-contiguous, `shape`) [i0..] = X[sum_d i_d * x_strides[d]].
- * Replaces PureTranspose.forward (pure_implementations.py:369-379). ndim <= 8. */
+ * Replaces PureTranspose.forward (pure_implementations.py:369-379), and
+ * PureSlice.forward (:619-693) with X pointing at the first selected element
+ * and x_strides = stride * step per axis. ndim <= 8. */
 int mi355x_permute_b32(const void* X, void* Y, int ndim, const int64_t* shape,
                        const int64_t* x_strides, void* stream);
+
+/* ONNX Cast between float, double, int32, int64, int8, uint8 and bool, one pass.
+ * Replaces PureCast.forward (pure_implementations.py:382-430: one map of
+ * `__output = __input`, i.e. the C conversion, which truncates toward zero
+ * from floating point to integers); to bool is `x != 0`.
+ * `from_type` / `to_type` are ONNX TensorProto data types (the values of the
+ * node's `to` attribute): 1 float, 2 uint8, 3 int8, 6 int32, 7 int64, 9 bool,
+ * 11 double. n elements, both buffers C-contiguous. */
+#define MI355X_TYPE_FLOAT 1
+#define MI355X_TYPE_UINT8 2
+#define MI355X_TYPE_INT8 3
+#define MI355X_TYPE_INT32 6
+#define MI355X_TYPE_INT64 7
+#define MI355X_TYPE_BOOL 9
+#define MI355X_TYPE_DOUBLE 11
+int mi355x_cast(const void* X, int from_type, void* Y, int to_type, int64_t n,
+                void* stream);
 
 #ifdef __cplusplus
 }

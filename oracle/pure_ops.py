@@ -328,6 +328,24 @@ def pow(X, Y):  # noqa: A001 (named after the ONNX op)
     return np.power(X, np.asarray(Y, dtype=X.dtype)).astype(X.dtype, copy=False)
 
 
+def cast(X, np_dtype):
+    """PureCast (pure_implementations.py:382-430): one map of ``__output = __input``, the C conversion
+    (floating point to integer truncates toward zero, as numpy's astype does for values in range)."""
+    return X.astype(np_dtype)
+
+
+def slice_(data, starts, ends, axes=None, steps=None):
+    """ONNX Slice; PureSlice (pure_implementations.py:619-693) is the axis-0, step-1 case
+    ``data[start:end:1, :]`` with ``end == INT64_MAX`` meaning "to the end". Python slicing already clamps
+    bounds the way the operator specifies."""
+    axes = list(range(len(starts))) if axes is None else list(axes)
+    steps = [1] * len(starts) if steps is None else list(steps)
+    index = [slice(None)] * data.ndim
+    for s, e, ax, st in zip(starts, ends, axes, steps):
+        index[int(ax)] = slice(int(s), int(e), int(st))
+    return np.ascontiguousarray(data[tuple(index)])
+
+
 def transpose(X, perm=None):
     """PureTranspose (pure_implementations.py:369-379)."""
     return np.ascontiguousarray(np.transpose(X, axes=perm))

@@ -244,8 +244,28 @@ def test_proto_reads_reference_fixture():
     data = open(os.path.join(GOLDEN_DIR, "slice.onnx"), "rb").read()
     assert proto.serialize_model(proto.parse_model(proto.serialize_model(m))) == proto.serialize_model(m)
     assert len(proto.serialize_model(m)) in (len(data), len(data) + 2)  # producer_name field is written empty
-    with pytest.raises(ValueError, match="Unsupported ONNX operator: 'Slice'"):
-        donnx.ONNXModel("slice", m)
+    model = donnx.ONNXModel("slice", m, fold_constants=False)       # imports and expands without a GPU
+    calls = [n for n, _ in model.expand().all_nodes_recursive() if isinstance(n, dace.KernelCall)]
+    assert [c.function for c in calls] == ["mi355x_permute_b32"] and calls[0].args[3].values == [1]
+    with pytest.raises(ValueError, match="Unsupported ONNX operator: 'NonZero'"):
+        bad = proto.parse_model(proto.serialize_model(m))
+        bad.graph.node[0].op_type = "NonZero"
+        donnx.ONNXModel("nonzero", bad)
+
+
+def test_reference_bert_subgraph_fixture_imports_and_folds():
+    """tests/onnx_files/reshape.onnx of the reference (Slice of the position embeddings, Cast of the target
+    shape, Reshape): imported as in tests/test_bert_subgraphs.py:29-32 with fold_constants=False -- the Reshape
+    target is then computed by the Cast node and the result's shape comes from the model's declaration -- and
+    with folding, which (tests/transformation/test_constant_folding.py:17-41) leaves only the data path."""
+    m = proto.load(os.path.join(GOLDEN_DIR, "reshape.onnx"))
+    assert [n.op_type for n in m.graph.node] == ["Slice", "Cast", "Reshape"] and not m.graph.input
+    unfolded = donnx.ONNXModel("bert_subgraph", m, fold_constants=False, fuse=False)
+    calls = [n.function for n, _ in unfolded.expand().all_nodes_recursive() if isinstance(n, dace.KernelCall)]
+    assert sorted(calls) == ["mi355x_cast", "mi355x_permute_b32"]
+    folded = donnx.ONNXModel("bert_subgraph_folded", m, fold_constants=True, fuse=False)
+    calls = [n.function for n, _ in folded.expand().all_nodes_recursive() if isinstance(n, dace.KernelCall)]
+    assert calls == []       # the Slice of a constant folds, the Cast folds, the Reshape is a view
 
 
 def test_proto_roundtrip_all_attribute_kinds():

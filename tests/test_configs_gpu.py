@@ -6,6 +6,7 @@ restatement for the convolution and the integer product) and from
 size-independent properties otherwise.
 """
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -16,7 +17,7 @@ import dace_onnx_amd.onnx as donnx
 from dace_onnx_amd.testing.graphs import bert_encoder_layer_model, conv_relu_model
 from dace_onnx_amd.onnx import proto
 from oracle import pure_ops as O
-from conftest import rel_err, FP32_REL_TOL
+from conftest import rel_err, FP32_REL_TOL, GOLDEN_DIR
 
 pytestmark = pytest.mark.gpu
 
@@ -401,3 +402,33 @@ def test_classifier_head_with_log_softmax_reductions_and_sum():
     assert rel_err(O.reduce_sum(logits, [1]), rs) < FP32_REL_TOL
     assert np.allclose(rmax, O.reduce_max(logits, [1]), rtol=1e-5) and np.allclose(rmin, O.reduce_min(logits, [0], 0), rtol=1e-5)
     assert rel_err(O.sum_(O.log_softmax(logits, axis=1), logits, O.log_softmax(logits, axis=1)), total) < FP32_REL_TOL
+
+
+# ----------------------------------------------------------------------------- the reference's ONNX file fixtures
+def test_reference_slice_fixture():
+    # tests/test_bert_subgraphs.py:17-26 of the reference, on its own data file
+    model = donnx.ONNXModel("slice_fixture", proto.load(os.path.join(GOLDEN_DIR, "slice.onnx")), fold_constants=False)
+    out = model(data=torch.ones(2, device="cuda"))
+    assert out.shape == (1, ) and out[0] == 1.0
+    out = model(data=torch.tensor([3.0, 7.0], device="cuda"))
+    assert out.tolist() == [3.0]
+
+
+@pytest.mark.parametrize("fold", [False, True])
+def test_reference_bert_subgraph_fixture(fold):
+    """tests/test_bert_subgraphs.py:29-52 and tests/transformation/test_constant_folding.py:17-41 of the
+    reference, on its own data file: a model without inputs (Slice of the position embeddings, Cast of the
+    target shape, Reshape); same result with and without constant folding; the saved Cast result equals the
+    shape weight."""
+    m = proto.load(os.path.join(GOLDEN_DIR, "reshape.onnx"))
+    weights = {t.name: np.asarray(t.array).reshape(t.dims) for t in m.graph.initializer}
+    saved = {}
+    model = donnx.ONNXModel(f"bert_subgraph_{fold}", m, fold_constants=fold, save_transients=None if fold else saved)
+    out = model()
+    emb = weights["bert/embeddings/position_embeddings:0"]
+    expected = O.slice_(emb, weights["const_slice__40"], weights["const_slice__41"]).reshape(1, 256, 768)
+    assert tuple(out.shape) == (1, 256, 768) and np.array_equal(np.asarray(out), expected)   # no inputs: numpy result
+    if not fold:
+        cast = saved["bertSLASHembeddingsSLASHReshape_4__42COLON0"]
+        assert cast.dtype == torch.int64
+        assert torch.equal(cast.type(torch.int32).cpu(), model.weights["bert/embeddings/Reshape_4/shape:0"].cpu())

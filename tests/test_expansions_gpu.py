@@ -13,6 +13,7 @@ import torch
 
 from dace_onnx_amd import _lib, sdfg as dace
 import dace_onnx_amd.onnx as donnx
+from dace_onnx_amd.onnx import proto
 from dace_onnx_amd.util import utils
 from oracle import pure_ops as O
 from conftest import rel_err, FP32_REL_TOL
@@ -397,6 +398,44 @@ def test_sum(count, shape):
     Y = np.zeros(shape, np.float32)
     donnx.ONNXSum(**{f"data_0__{i}": x for i, x in enumerate(xs)}, sum=Y)
     assert np.array_equal(O.sum_(*xs), Y)
+
+
+@pytest.mark.parametrize("src, dst", [(np.float32, np.int32), (np.float32, np.int64), (np.int64, np.float32),
+                                      (np.int32, np.int64), (np.int64, np.int32), (np.float32, np.float64),
+                                      (np.float64, np.float32), (np.float32, np.bool_), (np.int8, np.float32),
+                                      (np.uint8, np.int32), (np.float32, np.int8), (np.bool_, np.float32),
+                                      (np.float32, np.float32)])
+@pytest.mark.parametrize("n", [1, 1000, 70001])
+def test_cast(src, dst, n):
+    """PureCast (pure_implementations.py:382-430): the C conversion, element by element, exact."""
+    rng = np.random.default_rng(23)
+    X = (rng.normal(scale=40, size=n) * (rng.random(n) > 0.2)).astype(src)       # zeros included, for bool
+    Y = np.zeros(n, dst)
+    donnx.ONNXCast(input=X, output=Y, to=proto.np_dtype_to_tensor_dtype(np.dtype(dst)))
+    assert Y.dtype == np.dtype(dst) and np.array_equal(O.cast(X, dst), Y)
+
+
+@pytest.mark.parametrize("shape, starts, ends, axes, steps", [
+    ((2, ), [0], [1], [0], None),                                    # the reference's slice.onnx
+    ((512, 768), [0, 0], [256, 2 ** 63 - 1], None, None),            # the reference's reshape.onnx
+    ((20, 10, 6), [5], [2 ** 63 - 1], [0], [1]),                     # PureSlice's own case: axis 0, step 1, "to the end"
+    ((20, 10, 6), [1, 2], [18, -1], [0, 2], [3, 2]),
+    ((4, 9, 33), [-2, 30], [100, 3], [1, 2], [1, -4]),
+    ((7, 8), [6], [-100], [0], [-1]),
+    ((7, 8), [3], [3], [1], [1]),                                    # empty result
+    ((3, 130, 70), [1, 2], [129, 69], [-2, -1], [1, 1])])
+def test_slice(shape, starts, ends, axes, steps):
+    X = np.random.default_rng(24).normal(size=shape).astype(np.float32)
+    expected = O.slice_(X, starts, ends, axes, steps)
+    Y = np.full(expected.shape, np.nan, np.float32)
+    as_i64 = lambda v: None if v is None else np.array(v, dtype=np.int64)
+    kwargs = {k: as_i64(v) for k, v in (("starts", starts), ("ends", ends), ("axes", axes), ("steps", steps)) if v is not None}
+    donnx.ONNXSlice(data=X, output=Y, **kwargs)
+    assert np.array_equal(expected, Y)
+    Xi = np.arange(int(np.prod(shape)), dtype=np.int32).reshape(shape)          # any 4-byte element type
+    Yi = np.zeros(expected.shape, np.int32)
+    donnx.ONNXSlice(data=Xi, output=Yi, **kwargs)
+    assert np.array_equal(O.slice_(Xi, starts, ends, axes, steps), Yi)
 
 
 def test_pow():
