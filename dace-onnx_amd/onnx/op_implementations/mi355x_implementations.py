@@ -206,6 +206,94 @@ class MI355XMatMul(ONNXForward):
                           alpha=getattr(node, "_alpha", 1.0), epilogue=epi, offsets=MI355XMatMul._offsets(node))
 
 
+def _einsum_plan(equation, X0, X1, Y):
+    """A two-operand einsum as one strided batched GEMM: (plan, swapped) or None.
+
+    Letters are sorted into batch (in both inputs and the output), M (first input and output), N (second
+    input and output) and K (both inputs, not the output). All K letters must be walked as one axis by both
+    inputs; the last M and the last N letter are the GEMM's m and n, every other output letter is a batch
+    axis in which the operand that does not carry it is broadcast (stride 0) -- ``_BatchPlan`` folds such
+    axes back into M where the layout allows. The output's innermost letter must be an N letter (n stride 1);
+    when it is an M letter the two inputs change roles. Not expressible this way (and refused): ellipses,
+    a letter repeated inside one term, a letter that only one input carries and the output does not."""
+    eq = equation.replace(" ", "")
+    if "..." in eq or "->" not in eq:
+        return None
+    lhs, out = eq.split("->")
+    terms = lhs.split(",")
+    if len(terms) != 2 or any(not t.isalpha() for t in terms) or (out and not out.isalpha()):
+        return None
+    t0, t1 = terms
+    descs = {0: X0, 1: X1}
+    if len(t0) != len(X0.shape) or len(t1) != len(X1.shape) or len(out) != len(Y.shape):
+        return None
+    if len(set(t0)) != len(t0) or len(set(t1)) != len(t1) or len(set(out)) != len(out):
+        return None
+    size = {}
+    for term, d in ((t0, X0), (t1, X1), (out, Y)):
+        for letter, extent in zip(term, d.shape):
+            if size.setdefault(letter, extent) != extent:
+                return None
+    if not set(out) <= set(t0) | set(t1) or (set(t0) ^ set(t1)) - set(out):
+        return None
+    swapped = bool(out) and out[-1] in t0 and out[-1] not in t1      # innermost output letter must come from "B"
+    if swapped:
+        t0, t1 = t1, t0
+        descs = {0: X1, 1: X0}
+    stride = lambda term, d, letter: d.strides[term.index(letter)] if letter in term else 0
+    m_letters = [c for c in out if c in t0 and c not in t1]
+    n_letters = [c for c in out if c in t1 and c not in t0]
+    k_letters = [c for c in t0 if c in t1 and c not in out]
+    batch = [c for c in out if c not in m_letters[-1:] and c not in n_letters[-1:]]
+    # K letters as one axis of both inputs
+    K, a_sk, b_sk = 1, 0, 0
+    for c in reversed(k_letters):
+        sa, sb = stride(t0, descs[0], c), stride(t1, descs[1], c)
+        if K == 1:
+            a_sk, b_sk = sa, sb
+        elif sa != a_sk * K or sb != b_sk * K:
+            return None
+        K *= size[c]
+    m, n = (m_letters[-1:] or [None])[0], (n_letters[-1:] or [None])[0]
+    M, N = (size[m] if m else 1), (size[n] if n else 1)
+    shape_b = [size[c] for c in batch]
+    view = lambda term, d, tail_shape, tail: dace.Array(Y.dtype, shape_b + tail_shape,
+                                                         [stride(term, d, c) for c in batch] + tail)
+    A = view(t0, descs[0], [M, K], [stride(t0, descs[0], m) if m else 0, a_sk])
+    B = view(t1, descs[1], [K, N], [b_sk, stride(t1, descs[1], n) if n else 0])
+    C = view(out, Y, [M, N], [stride(out, Y, m) if m else 0, stride(out, Y, n) if n else 1])
+    plan = _BatchPlan(A, B, C)
+    return (plan, swapped) if plan.ok else None
+
+
+@op_implementation(op="Einsum", name=IMPLEMENTATION_NAME)
+class MI355XEinsum(ONNXForward):
+    """Two-operand fp32 contractions on the MFMA GEMM kernel, nothing copied or transposed (the reference
+    lowers Einsum -- and through it every MatMul -- to DaCe's einsum SDFG: PureEinsum, :238-267)."""
+
+    @staticmethod
+    def _plan(node, state, sdfg):
+        conns = sorted((c for c in node.in_connectors if c.startswith("Inputs__")), key=lambda c: int(c[len("Inputs__"):]))
+        if len(conns) != 2 or not node.equation:
+            return None
+        X0, X1 = (in_desc_with_name(node, state, sdfg, c) for c in conns)
+        Y = out_desc_with_name(node, state, sdfg, "Output")
+        if not _is_f32(X0, X1, Y) or not _contig(Y):
+            return None
+        equation = node.equation.decode() if isinstance(node.equation, bytes) else node.equation
+        found = _einsum_plan(equation, X0, X1, Y)
+        return None if found is None else (found[0], conns[::-1] if found[1] else conns)
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        return MI355XEinsum._plan(node, state, sdfg) is not None
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        plan, (a_conn, b_conn) = MI355XEinsum._plan(node, state, sdfg)
+        return _gemm_call(node, state, plan, a_conn, b_conn, "Output")
+
+
 @op_implementation(op="Gemm", name=IMPLEMENTATION_NAME)
 class MI355XGemm(ONNXForward):
     """``Y = alpha * A' B' + beta * C``. transA / transB are strides; ``C`` is

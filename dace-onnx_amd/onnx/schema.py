@@ -171,6 +171,9 @@ SCHEMAS: typing.List[ONNXSchema] = [
                [ONNXParameter("output", "T")], (),
                [ONNXTypeConstraint("T", _ANY), ONNXTypeConstraint("Tind", [dace.int32, dace.int64])],
                "data[starts:ends:steps] along `axes` (numpy slicing semantics, bounds clamped)."),
+    ONNXSchema("Einsum", 12, [ONNXParameter("Inputs", "T", ONNXParameterType.Variadic)], [ONNXParameter("Output", "T")],
+               [ONNXAttribute("equation", _A.String, required=True)],
+               [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64])], "Einstein summation."),
     ONNXSchema("Sum", 8, [ONNXParameter("data_0", "T", ONNXParameterType.Variadic)], [ONNXParameter("sum", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS)], "Elementwise sum of the inputs."),
 ]

@@ -135,6 +135,18 @@ def _infer_node(node, shapes, types, constants):
                 raise ShapeInferenceError(f"Slice '{node.name}': input '{name}' must be a constant initializer")
             idx.append([int(v) for v in constants[name].ravel()] if name else None)
         return [(tuple(c for _, _, c in slice_ranges(ins[0], *idx)), tys[0])]
+    if op == "Einsum":
+        eq = a["equation"].decode() if isinstance(a["equation"], bytes) else a["equation"]
+        eq = eq.replace(" ", "")
+        if "..." in eq or "->" not in eq:
+            raise ShapeInferenceError(f"Einsum '{node.name}': only explicit equations without ellipsis ('{eq}')")
+        lhs, out = eq.split("->")
+        size = {}
+        for term, shp in zip(lhs.split(","), ins):
+            if len(term) != len(shp):
+                raise ShapeInferenceError(f"Einsum '{node.name}': term '{term}' does not match a rank-{len(shp)} input")
+            size.update(zip(term, shp))
+        return [(tuple(size[c] for c in out), tys[0])]
     if op == "Sum":
         return [(tuple(np.broadcast_shapes(*ins)), tys[0])]
     if op in ("ReduceMean", "ReduceSum", "ReduceMax", "ReduceMin"):

@@ -328,6 +328,12 @@ def pow(X, Y):  # noqa: A001 (named after the ONNX op)
     return np.power(X, np.asarray(Y, dtype=X.dtype)).astype(X.dtype, copy=False)
 
 
+def einsum(equation, *operands):
+    """PureEinsum (pure_implementations.py:238-267) lowers to DaCe's einsum SDFG; numpy's einsum is the
+    comparator of the reference's own test (tests/pure_expansions/test_expansions.py:456-473)."""
+    return np.einsum(equation, *operands)
+
+
 def cast(X, np_dtype):
     """PureCast (pure_implementations.py:382-430): one map of ``__output = __input``, the C conversion
     (floating point to integer truncates toward zero, as numpy's astype does for values in range)."""

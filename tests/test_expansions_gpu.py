@@ -438,6 +438,38 @@ def test_slice(shape, starts, ends, axes, steps):
     assert np.array_equal(O.slice_(Xi, starts, ends, axes, steps), Yi)
 
 
+@pytest.mark.parametrize("equation, shapes", [
+    ("bij ,jk -> bik", [(5, 4, 3), (3, 2)]),                 # tests/pure_expansions/test_expansions.py:456-473 (there in fp64)
+    ("ik,kj->ij", [(33, 20), (20, 48)]),
+    ("bhqd,bhkd->bhqk", [(2, 3, 16, 8), (2, 3, 20, 8)]),     # Q K^T
+    ("bhqk,bhkd->bhqd", [(2, 3, 16, 20), (2, 3, 20, 8)]),    # P V
+    ("bqhd,bkhd->bhqk", [(2, 16, 3, 8), (2, 20, 3, 8)]),     # heads not split out beforehand
+    ("bik,jk->bij", [(4, 10, 12), (7, 12)]),                 # Linear: x W^T
+    ("ij,bjk->bik", [(6, 5), (3, 5, 8)]),                    # shared left operand
+    ("bij,bjk->bki", [(3, 6, 5), (3, 5, 8)]),                # transposed result: the inputs change roles
+    ("abc,cd->abd", [(2, 3, 4), (4, 4)]),
+    ("ijk,jkl->il", [(6, 4, 5), (4, 5, 7)]),                 # two contracted letters walked as one axis
+    ("i,j->ij", [(9, ), (12, )]),                            # outer product (K = 1)
+    ("bi,bi->b", [(6, 40), (6, 40)])])                       # batched dot product (M = N = 1)
+def test_einsum(equation, shapes):
+    rng = np.random.default_rng(25)
+    xs = [rng.normal(size=s).astype(np.float32) for s in shapes]
+    expected = O.einsum(equation, *[x.astype(np.float64) for x in xs])
+    Y = np.zeros(expected.shape, np.float32)
+    donnx.ONNXEinsum(Inputs__0=xs[0], Inputs__1=xs[1], Output=Y, equation=equation)
+    assert rel_err(expected, Y) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("equation, shapes", [("ii->i", [(4, 4)]), ("ij,jk,kl->il", [(2, 3), (3, 4), (4, 5)]),
+                                              ("ij,jk->i", [(2, 3), (3, 4)]), ("...ij,jk->...ik", [(2, 2, 3), (3, 4)]),
+                                              ("ijk,kjl->il", [(6, 4, 5), (5, 4, 7)])])
+def test_einsum_refuses_what_one_gemm_cannot_do(equation, shapes):
+    xs = [np.zeros(s, np.float32) for s in shapes]
+    out_shape = np.einsum(equation, *xs).shape
+    with pytest.raises(donnx.ExpansionRefused):
+        donnx.ONNXEinsum(**{f"Inputs__{i}": x for i, x in enumerate(xs)}, Output=np.zeros(out_shape, np.float32), equation=equation)
+
+
 def test_pow():
     rng = np.random.default_rng(16)
     X = rng.normal(size=(8, 16, 64)).astype(np.float32)
