@@ -15,7 +15,19 @@ Softmax             PureSoftmax, pure_implementations.py:346-366
 LayerNormalization  (exporter decomposition, pure_implementations.py:97-109 etc.)
 Add/Sub/Mul/Div     python_pure_op_implementation, pure_implementations.py:77-94
 Relu, Erf, Sqrt     pure_implementations.py:462-474, 112-127, 41-56
+Pow                 PurePow, pure_implementations.py:59-74
+Log, Reciprocal,    PureLog :23-38, PureReciprocal :275-293, Tanh :296-298,
+Tanh, Softplus,     Softplus :696-698, PureSigmoid :701-712
+Sigmoid
+Exp, Neg, Abs       (ONNX Runtime only in the reference)
 Gelu                (exporter decomposition Div, Erf, Add, Mul, Mul)
+ReduceMean/Sum/     PureReduceMean :97-109, PureReduceSum / Max / Min :301-343
+Max/Min
+LogSoftmax          PureLogSoftmax, pure_implementations.py:594-616
+Sum                 PureSum, pure_implementations.py:529-591
+Einsum              PureEinsum, pure_implementations.py:238-267
+Cast                PureCast, pure_implementations.py:382-430
+Slice               PureSlice, pure_implementations.py:619-693
 Transpose           PureTranspose, pure_implementations.py:369-379
 Reshape, Flatten    PureReshape / PureFlatten, pure_implementations.py:477-526
 Identity            pure_implementations.py:270-272
