@@ -49,6 +49,8 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
                                     _c_i64_p, _c_i64_p, _c_i64_p, _c_i64_p, _f32, _vp]),
     "mi355x_layernorm_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "mi355x_reduce_mean_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_maxpool2d_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "mi355x_batchnorm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),
     "mi355x_cast": (_int, [_vp, _int, _vp, _int, _i64, _vp]),
     "mi355x_reduce_f32": (_int, [_int, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_log_softmax_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),

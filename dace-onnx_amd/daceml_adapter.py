@@ -135,7 +135,8 @@ def register(ops: typing.Optional[typing.Iterable[str]] = None) -> typing.List[s
     registered = []
     for op in (ops or ["MatMul", "Gemm", "Conv", "MatMulInteger", "Softmax", "Add", "Sub", "Mul", "Div", "Pow", "Relu", "Erf",
                        "Sqrt", "Log", "Tanh", "Sigmoid", "Softplus", "Reciprocal", "Exp", "Neg", "Abs", "ReduceMean", "ReduceSum",
-                       "ReduceMax", "ReduceMin", "LogSoftmax", "Sum", "Cast", "Slice", "Einsum", "Transpose"]):
+                       "ReduceMax", "ReduceMin", "LogSoftmax", "Sum", "Cast", "Slice", "Einsum", "MaxPool", "GlobalAveragePool",
+                       "BatchNormalization", "Transpose"]):
         dace_node = getattr(donnx, "ONNX" + op, None)
         if dace_node is None:
             continue

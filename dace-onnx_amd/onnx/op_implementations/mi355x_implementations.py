@@ -449,6 +449,95 @@ class MI355XConv(ONNXForward):
             N, C, H, Wd, M, KH, KW, I64Array(pads), I64Array(strides), I64Array(dil), epi, Stream()])
 
 
+@op_implementation(op="MaxPool", name=IMPLEMENTATION_NAME)
+class MI355XMaxPool(ONNXForward):
+    """2-D max pooling with pads, strides and dilations (floor output size, no ``Indices`` output).
+    PureMaxPool2D (img_op_implementations.py:28-161) refuses pads and dilations."""
+
+    @staticmethod
+    def _geometry(node, X):
+        if node.kernel_shape is None or len(node.kernel_shape) != 2 or len(X.shape) != 4:
+            return None
+        window = dace.Array(X.dtype, [1, 1] + [int(k) for k in node.kernel_shape])
+        geom = _conv_geometry(node, X, window)
+        if geom is None:
+            return None
+        pads, strides, dil, oh, ow = geom
+        eff = [(window.shape[2] - 1) * dil[0] + 1, (window.shape[3] - 1) * dil[1] + 1]
+        if max(pads[0], pads[2]) >= eff[0] or max(pads[1], pads[3]) >= eff[1]:
+            return None                 # a window entirely inside the padding has no maximum
+        return pads, strides, dil, oh, ow
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "X")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        if _has_output(node, state, "Indices") or (node.ceil_mode or 0) != 0 or (node.storage_order or 0) != 0:
+            return False
+        if not _is_f32(X, Y) or not _contig(X, Y):
+            return False
+        geom = MI355XMaxPool._geometry(node, X)
+        return geom is not None and tuple(Y.shape) == (X.shape[0], X.shape[1], geom[3], geom[4])
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "X")
+        pads, strides, dil, _, _ = MI355XMaxPool._geometry(node, X)
+        return kernel_call_for_node(node, state, "mi355x_maxpool2d_f32", [
+            Ptr("X"), Ptr("Y"), X.shape[0], X.shape[1], X.shape[2], X.shape[3], int(node.kernel_shape[0]),
+            int(node.kernel_shape[1]), I64Array(pads), I64Array(strides), I64Array(dil), Stream()])
+
+
+@op_implementation(op="GlobalAveragePool", name=IMPLEMENTATION_NAME)
+class MI355XGlobalAveragePool(ONNXForward):
+    """Mean over the spatial axes (GlobalAveragePool, img_op_implementations.py:410-412): the row mean of
+    ``[N * C, H * W]``."""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        X = in_desc_with_name(node, state, sdfg, "X")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        return _is_f32(X, Y) and _contig(X, Y) and len(X.shape) >= 3 and prod(X.shape[2:]) >= 1 and \
+            tuple(Y.shape) == tuple(X.shape[:2]) + (1, ) * (len(X.shape) - 2)
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "X")
+        return kernel_call_for_node(node, state, "mi355x_reduce_mean_f32",
+                                    [Ptr("X"), Ptr("Y"), prod(X.shape[:2]), prod(X.shape[2:]), 1, Stream()])
+
+
+@op_implementation(op="BatchNormalization", name=IMPLEMENTATION_NAME)
+class MI355XBatchNormalization(ONNXForward):
+    """Inference form: the stored mean and variance are used, only ``Y`` is produced. (The reference's
+    PureBatchNormalization, img_op_implementations.py:329-407, is the training form -- batch statistics and
+    running-mean update -- and is not provided here; a node with the training outputs is refused.)"""
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        if any(_has_output(node, state, c) for c in ("out_mean", "out_var", "saved_mean", "saved_var")):
+            return False
+        X = in_desc_with_name(node, state, sdfg, "X")
+        Y = out_desc_with_name(node, state, sdfg, "Y")
+        if not _is_f32(X, Y) or not _contig(X, Y) or len(X.shape) < 2 or tuple(X.shape) != tuple(Y.shape):
+            return False
+        for conn in ("scale", "B", "mean", "var"):
+            if not _has_input(node, state, conn):
+                return False
+            d = in_desc_with_name(node, state, sdfg, conn)
+            if not _is_f32(d) or not _contig(d) or tuple(d.shape) != (X.shape[1], ):
+                return False
+        return True
+
+    @staticmethod
+    def forward(node, state: SDFGState, sdfg: SDFG):
+        X = in_desc_with_name(node, state, sdfg, "X")
+        eps = 1e-5 if node.epsilon is None else float(node.epsilon)
+        return kernel_call_for_node(node, state, "mi355x_batchnorm_f32", [
+            Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("mean"), Ptr("var"), Ptr("Y"), X.shape[0], X.shape[1],
+            prod(X.shape[2:]), eps, Stream()])
+
+
 @op_implementation(op="MatMulInteger", name=IMPLEMENTATION_NAME)
 class MI355XMatMulInteger(ONNXForward):
     """int8 x int8 -> int32 on int8 MFMA, bit-exact, scalar zero points read on

@@ -174,6 +174,20 @@ SCHEMAS: typing.List[ONNXSchema] = [
     ONNXSchema("Einsum", 12, [ONNXParameter("Inputs", "T", ONNXParameterType.Variadic)], [ONNXParameter("Output", "T")],
                [ONNXAttribute("equation", _A.String, required=True)],
                [ONNXTypeConstraint("T", _FLOATS + [dace.int32, dace.int64])], "Einstein summation."),
+    ONNXSchema("MaxPool", 12, [ONNXParameter("X", "T")], [ONNXParameter("Y", "T"), ONNXParameter("Indices", "I", _O)],
+               [ONNXAttribute("auto_pad", _A.String, "NOTSET"), ONNXAttribute("ceil_mode", _A.Int, 0),
+                ONNXAttribute("dilations", _A.Ints), ONNXAttribute("kernel_shape", _A.Ints, required=True),
+                ONNXAttribute("pads", _A.Ints), ONNXAttribute("storage_order", _A.Int, 0), ONNXAttribute("strides", _A.Ints)],
+               [ONNXTypeConstraint("T", _FLOATS + [dace.int8, dace.uint8]), ONNXTypeConstraint("I", [dace.int64])],
+               "Max pooling over sliding windows."),
+    _unary("GlobalAveragePool", 1, "X", "Y", doc="Mean over the spatial axes."),
+    ONNXSchema("BatchNormalization", 9,
+               [ONNXParameter("X", "T"), ONNXParameter("scale", "T"), ONNXParameter("B", "T"), ONNXParameter("mean", "T"),
+                ONNXParameter("var", "T")],
+               [ONNXParameter("Y", "T"), ONNXParameter("out_mean", "T", _O), ONNXParameter("out_var", "T", _O),
+                ONNXParameter("saved_mean", "T", _O), ONNXParameter("saved_var", "T", _O)],
+               [ONNXAttribute("epsilon", _A.Float, 1e-5), ONNXAttribute("momentum", _A.Float, 0.9)],
+               [ONNXTypeConstraint("T", _FLOATS)], "Batch normalization."),
     ONNXSchema("Sum", 8, [ONNXParameter("data_0", "T", ONNXParameterType.Variadic)], [ONNXParameter("sum", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS)], "Elementwise sum of the inputs."),
 ]

@@ -135,6 +135,28 @@ def _infer_node(node, shapes, types, constants):
                 raise ShapeInferenceError(f"Slice '{node.name}': input '{name}' must be a constant initializer")
             idx.append([int(v) for v in constants[name].ravel()] if name else None)
         return [(tuple(c for _, _, c in slice_ranges(ins[0], *idx)), tys[0])]
+    if op == "BatchNormalization":
+        return [(ins[0], tys[0])] + [((ins[0][1], ), tys[0])] * (len(node.output) - 1)
+    if op == "GlobalAveragePool":
+        return [(tuple(ins[0][:2]) + (1, ) * (len(ins[0]) - 2), tys[0])]
+    if op == "MaxPool":
+        X = ins[0]
+        nsp = len(X) - 2
+        kernel = a.get("kernel_shape")
+        strides = a.get("strides") or [1] * nsp
+        dil = a.get("dilations") or [1] * nsp
+        auto_pad = a.get("auto_pad", "NOTSET")
+        auto_pad = auto_pad.decode() if isinstance(auto_pad, bytes) else auto_pad
+        if a.get("ceil_mode", 0):
+            raise ShapeInferenceError(f"MaxPool '{node.name}': ceil_mode is not supported")
+        out = []
+        for i in range(nsp):
+            if auto_pad in ("SAME_UPPER", "SAME_LOWER"):
+                out.append(-(-X[2 + i] // strides[i]))
+            else:
+                pads = (a.get("pads") or [0] * (2 * nsp)) if auto_pad == "NOTSET" else [0] * (2 * nsp)
+                out.append(_conv_out(X[2 + i], kernel[i], strides[i], dil[i], pads[i], pads[i + nsp]))
+        return [((X[0], X[1]) + tuple(out), tys[0])] + [((X[0], X[1]) + tuple(out), TensorProto.INT64)] * (len(node.output) - 1)
     if op == "Einsum":
         eq = a["equation"].decode() if isinstance(a["equation"], bytes) else a["equation"]
         eq = eq.replace(" ", "")

@@ -104,6 +104,24 @@ int mi355x_conv2d_f32(const float* X, const float* W, const float* bias, float* 
                       const int64_t* pads, const int64_t* strides,
                       const int64_t* dilations, int epilogue, void* stream);
 
+/* ONNX MaxPool, 2-D, fp32, NCHW: Y[n,c,oh,ow] = max over the KH x KW window at
+ * (oh * strides[0] - pads[0] + kh * dilations[0], ow * strides[1] - pads[1] + kw * dilations[1]);
+ * positions in the padding do not take part. pads = {top, left, bottom, right}, floor output size
+ * (ceil_mode 0). Replaces PureMaxPool2D.forward (img_op_implementations.py:28-161), which accepts
+ * neither pads nor dilations. */
+int mi355x_maxpool2d_f32(const float* X, float* Y, int64_t N, int64_t C, int64_t H, int64_t W,
+                         int64_t KH, int64_t KW, const int64_t* pads, const int64_t* strides,
+                         const int64_t* dilations, void* stream);
+
+/* ONNX BatchNormalization in inference form, fp32, X and Y are [N, C, HW]:
+ * Y = (X - mean[c]) * (1 / sqrt(var[c] + eps)) * scale[c] + B[c], the arithmetic of
+ * PureBatchNormalization.forward (img_op_implementations.py:362-375) with the stored statistics in
+ * place of the batch's (the reference expands the training form only and leaves inference to ONNX
+ * Runtime). */
+int mi355x_batchnorm_f32(const float* X, const float* scale, const float* B, const float* mean,
+                         const float* var, float* Y, int64_t N, int64_t C, int64_t HW, float eps,
+                         void* stream);
+
 /* ONNX MatMulInteger, int8 x int8 -> int32 on int8 MFMA, bit-exact.
  *   Y[m,n] = sum_k (A[m,k] - a_zero_point) * (B[k,n] - b_zero_point)
  * The reference has no expansion of its own for this node: the generated class

@@ -328,6 +328,41 @@ def pow(X, Y):  # noqa: A001 (named after the ONNX op)
     return np.power(X, np.asarray(Y, dtype=X.dtype)).astype(X.dtype, copy=False)
 
 
+def maxpool2d(X, kernel_shape, strides=(1, 1), pads=(0, 0, 0, 0), dilations=(1, 1)):
+    """PureMaxPool2D (img_op_implementations.py:28-161): Y starts at the smallest value and every window element
+    is folded in with max. The reference refuses pads and dilations; here padded positions simply do not take
+    part (ONNX pads MaxPool with -inf)."""
+    N, C, H, W = X.shape
+    KH, KW = kernel_shape
+    eh, ew = (KH - 1) * dilations[0] + 1, (KW - 1) * dilations[1] + 1
+    OH = (H + pads[0] + pads[2] - eh) // strides[0] + 1
+    OW = (W + pads[1] + pads[3] - ew) // strides[1] + 1
+    Xp = np.full((N, C, H + pads[0] + pads[2], W + pads[1] + pads[3]), -np.inf, dtype=X.dtype)
+    Xp[:, :, pads[0]:pads[0] + H, pads[1]:pads[1] + W] = X
+    Y = np.full((N, C, OH, OW), -np.inf, dtype=X.dtype)
+    for kh in range(KH):
+        for kw in range(KW):
+            h0, w0 = kh * dilations[0], kw * dilations[1]
+            window = Xp[:, :, h0:h0 + (OH - 1) * strides[0] + 1:strides[0], w0:w0 + (OW - 1) * strides[1] + 1:strides[1]]
+            Y = np.maximum(Y, window)
+    return Y
+
+
+def global_average_pool(X):
+    """GlobalAveragePool (img_op_implementations.py:410-412): mean over axes 2 and 3, kept as size-1 axes."""
+    return np.mean(X, axis=tuple(range(2, X.ndim)), keepdims=True).astype(X.dtype, copy=False)
+
+
+def batch_normalization(X, scale, B, mean, var, epsilon=1e-5):
+    """Inference BatchNormalization in the arithmetic order of PureBatchNormalization
+    (img_op_implementations.py:362-375), with the stored statistics where the training form uses the batch's:
+    (X - mean) * (1 / sqrt(var + eps)) * scale + B, statistics broadcast as [C, 1, ...]."""
+    bshape = (1, -1) + (1, ) * (X.ndim - 2)
+    one = np.asarray(1.0, dtype=X.dtype)
+    normalized = (X - mean.reshape(bshape)) * (one / np.sqrt(var.reshape(bshape) + np.asarray(epsilon, dtype=X.dtype)))
+    return (normalized * scale.reshape(bshape) + B.reshape(bshape)).astype(X.dtype, copy=False)
+
+
 def einsum(equation, *operands):
     """PureEinsum (pure_implementations.py:238-267) lowers to DaCe's einsum SDFG; numpy's einsum is the
     comparator of the reference's own test (tests/pure_expansions/test_expansions.py:456-473)."""

@@ -470,6 +470,47 @@ def test_einsum_refuses_what_one_gemm_cannot_do(equation, shapes):
         donnx.ONNXEinsum(**{f"Inputs__{i}": x for i, x in enumerate(xs)}, Output=np.zeros(out_shape, np.float32), equation=equation)
 
 
+@pytest.mark.parametrize("shape, kernel, strides, pads, dil", [
+    ((5, 3, 10, 10), (2, 2), (2, 2), None, None),                       # LeNet-style pooling
+    ((2, 64, 112, 112), (3, 3), (2, 2), (1, 1, 1, 1), None),             # ResNet stem
+    ((1, 2, 9, 11), (3, 2), (1, 2), (1, 0, 2, 1), None), ((3, 4, 17, 13), (2, 3), (1, 1), (0, 1, 0, 1), (2, 2)),
+    ((2, 3, 7, 7), (7, 7), None, None, None)])
+def test_maxpool(shape, kernel, strides, pads, dil):
+    """PureMaxPool2D (img_op_implementations.py:28-161), plus pads / dilations: exact."""
+    X = np.random.default_rng(27).normal(size=shape).astype(np.float32)
+    expected = O.maxpool2d(X, kernel, strides or (1, 1), pads or (0, 0, 0, 0), dil or (1, 1))
+    Y = np.zeros(expected.shape, np.float32)
+    attrs = {k: list(v) for k, v in (("strides", strides), ("pads", pads), ("dilations", dil)) if v is not None}
+    donnx.ONNXMaxPool(X=X, Y=Y, kernel_shape=list(kernel), **attrs)
+    assert np.array_equal(expected, Y)
+
+
+def test_maxpool_nan_and_refusals():
+    X = np.random.default_rng(28).normal(size=(1, 1, 6, 6)).astype(np.float32)
+    X[0, 0, 2, 3] = np.nan
+    Y = np.zeros((1, 1, 3, 3), np.float32)
+    donnx.ONNXMaxPool(X=X, Y=Y, kernel_shape=[2, 2], strides=[2, 2])
+    assert np.array_equal(O.maxpool2d(X, (2, 2), (2, 2)), Y, equal_nan=True) and np.isnan(Y).sum() == 1
+    with pytest.raises(donnx.ExpansionRefused):
+        donnx.ONNXMaxPool(X=X, Y=np.zeros((1, 1, 3, 3), np.float32), kernel_shape=[2, 2], strides=[2, 2], ceil_mode=1)
+
+
+@pytest.mark.parametrize("shape", [(32, 64, 56, 56), (2, 3, 7, 5), (4, 16, 1, 1), (1, 5, 33)])
+def test_global_average_pool_and_batch_normalization(shape):
+    rng = np.random.default_rng(29)
+    X = rng.normal(1.0, 2.0, size=shape).astype(np.float32)
+    Y = np.zeros(shape[:2] + (1, ) * (len(shape) - 2), np.float32)
+    donnx.ONNXGlobalAveragePool(X=X, Y=Y)
+    assert rel_err(O.global_average_pool(X.astype(np.float64)), Y) < FP32_REL_TOL
+    C = shape[1]
+    scale, b, mean = (rng.normal(size=C).astype(np.float32) for _ in range(3))
+    var = rng.uniform(0.5, 2.0, size=C).astype(np.float32)
+    Z = np.zeros_like(X)
+    donnx.ONNXBatchNormalization(X=X, scale=scale, B=b, mean=mean, var=var, Y=Z, epsilon=1e-3)
+    expected = O.batch_normalization(X, scale, b, mean, var, 1e-3)
+    assert np.allclose(Z, expected, rtol=1e-5, atol=1e-5) and rel_err(expected, Z) < 1e-6
+
+
 def test_pow():
     rng = np.random.default_rng(16)
     X = rng.normal(size=(8, 16, 64)).astype(np.float32)

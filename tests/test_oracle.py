@@ -240,6 +240,44 @@ def test_reductions_log_softmax_sum_closed_forms():
     assert np.array_equal(O.sum_(a, b, c), (a + b) + c) and np.array_equal(O.sum_(a), a)
 
 
+@pytest.mark.parametrize("kernel, strides, pads, dil", [((2, 2), (2, 2), (0, 0, 0, 0), (1, 1)), ((3, 3), (2, 2), (1, 1, 1, 1), (1, 1)),
+                                                        ((3, 2), (1, 2), (1, 0, 2, 1), (1, 1)), ((2, 3), (1, 1), (0, 1, 0, 1), (2, 2))])
+def test_maxpool_global_average_pool_batchnorm_vs_torch(kernel, strides, pads, dil):
+    """MaxPool against torch's max_pool2d (symmetric pads) and a brute-force window loop (any pads);
+    GlobalAveragePool and inference BatchNormalization against torch and their closed forms."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(26)
+    x = rng.normal(size=(2, 3, 9, 11)).astype(np.float32)
+    got = O.maxpool2d(x, kernel, strides, pads, dil)
+    if pads[0] == pads[2] and pads[1] == pads[3]:
+        ref = F.max_pool2d(torch.from_numpy(x), kernel, strides, (pads[0], pads[1]), dil).numpy()
+        assert np.array_equal(got, ref)
+    eh, ew = (kernel[0] - 1) * dil[0] + 1, (kernel[1] - 1) * dil[1] + 1
+    for oh in range(got.shape[2]):
+        for ow in range(got.shape[3]):
+            best = np.full((2, 3), -np.inf, np.float32)
+            for kh in range(kernel[0]):
+                for kw in range(kernel[1]):
+                    ih, iw = oh * strides[0] - pads[0] + kh * dil[0], ow * strides[1] - pads[1] + kw * dil[1]
+                    if 0 <= ih < 9 and 0 <= iw < 11:
+                        best = np.maximum(best, x[:, :, ih, iw])
+            assert np.array_equal(got[:, :, oh, ow], best)
+    assert got.shape[2:] == ((9 + pads[0] + pads[2] - eh) // strides[0] + 1, (11 + pads[1] + pads[3] - ew) // strides[1] + 1)
+    gap = O.global_average_pool(x)
+    assert gap.shape == (2, 3, 1, 1) and np.allclose(gap, F.adaptive_avg_pool2d(torch.from_numpy(x), 1).numpy(), atol=1e-6)
+    scale, b, mean = (rng.normal(size=3).astype(np.float32) for _ in range(3))
+    var = rng.uniform(0.5, 2.0, size=3).astype(np.float32)
+    bn = O.batch_normalization(x, scale, b, mean, var, 1e-5)
+    ref = F.batch_norm(torch.from_numpy(x), torch.from_numpy(mean), torch.from_numpy(var), torch.from_numpy(scale),
+                       torch.from_numpy(b), training=False, eps=1e-5).numpy()
+    assert np.allclose(bn, ref, rtol=1e-5, atol=1e-6)
+    # identity statistics leave x unchanged up to eps; zero scale gives the bias
+    ident = O.batch_normalization(x, np.ones(3, np.float32), np.zeros(3, np.float32), np.zeros(3, np.float32), np.ones(3, np.float32), 0.0)
+    assert np.array_equal(ident, x)
+    assert np.array_equal(O.batch_normalization(x, np.zeros(3, np.float32), b, mean, var)[0, :, 0, 0], b)
+
+
 def test_pow_and_reduce_mean_closed_forms():
     rng = np.random.default_rng(21)
     x = rng.normal(size=(3, 5, 7)).astype(np.float32)
