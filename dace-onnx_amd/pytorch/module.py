@@ -167,6 +167,25 @@ def _convert(g, m, prefix, x, shape):
         oh = (shape[2] + 2 * ph - dh * (kh - 1) - 1) // sh + 1
         ow = (shape[3] + 2 * pw - dw * (kw - 1) - 1) // sw + 1
         return y, [shape[0], m.out_channels, oh, ow]
+    if isinstance(m, nn.BatchNorm2d):
+        if m.training or not m.track_running_stats or not m.affine or len(shape) != 4:
+            raise UnsupportedModule("BatchNorm2d: eval() mode with running statistics and affine parameters, NCHW input")
+        ins = [x, g.param(m.weight, prefix + "weight"), g.param(m.bias, prefix + "bias"),
+               g.param(m.running_mean, prefix + "running_mean"), g.param(m.running_var, prefix + "running_var")]
+        return g.node("BatchNormalization", ins, prefix + "out", epsilon=float(m.eps), momentum=float(1.0 - (m.momentum or 0.1))), shape
+    if isinstance(m, nn.MaxPool2d):
+        if m.ceil_mode or m.return_indices or len(shape) != 4:
+            raise UnsupportedModule("MaxPool2d: floor output size, no indices, NCHW input")
+        (kh, kw), (ph, pw), (dh, dw) = _pair(m.kernel_size), _pair(m.padding), _pair(m.dilation)
+        sh, sw = _pair(m.stride if m.stride is not None else m.kernel_size)
+        y = g.node("MaxPool", [x], prefix + "out", kernel_shape=[kh, kw], pads=[ph, pw, ph, pw], strides=[sh, sw], dilations=[dh, dw])
+        oh = (shape[2] + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+        ow = (shape[3] + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+        return y, [shape[0], shape[1], oh, ow]
+    if isinstance(m, nn.AdaptiveAvgPool2d):
+        if _pair(m.output_size) != (1, 1) or len(shape) != 4:
+            raise UnsupportedModule("AdaptiveAvgPool2d(1) only (GlobalAveragePool)")
+        return g.node("GlobalAveragePool", [x], prefix + "out"), [shape[0], shape[1], 1, 1]
     if isinstance(m, nn.ReLU):
         return g.node("Relu", [x], prefix + "out"), shape
     if isinstance(m, nn.GELU):

@@ -191,6 +191,77 @@ def _fuse_pad_conv(sdfg: SDFG, state: SDFGState) -> int:
     return fused
 
 
+def _fold_batchnorm_into_conv(sdfg: SDFG, state: SDFGState) -> int:
+    """Conv with constant weights whose only reader is an inference ``BatchNormalization`` with constant
+    parameters: the per-channel affine map moves into the convolution, ``W'[oc] = W[oc] * a[oc]`` and
+    ``bias' = (bias - mean) * a + B`` with ``a = scale / sqrt(var + eps)``, computed once at graph-preparation
+    time (the folded copies are new weights; the originals stay untouched). The reference has no counterpart:
+    its BatchNormalization expansion is the training form (``img_op_implementations.py:329-407``) and an
+    exported eval() network runs this pair as two ONNX Runtime nodes."""
+    model = getattr(sdfg, "_parent_onnx_model", None)
+    if model is None:
+        return 0
+    import torch
+    from ..onnx.onnx_importer import clean_onnx_name
+    by_clean = {clean_onnx_name(k): k for k in model.weights}
+
+    def constant(node, conn):
+        e = _in_edge(state, node, conn)
+        if e is None or not isinstance(e.src, AccessNode) or e.src.data not in by_clean or state.in_edges(e.src):
+            return None
+        w = model.weights[by_clean[e.src.data]]
+        return (e, w) if w.dtype == torch.float32 else None
+
+    folded = 0
+    for conv in list(state.nodes()):
+        if not _is_op(conv, "Conv") or _in_edge(state, conv, "_residual") is not None or getattr(conv, "_activation", None):
+            continue
+        y_e = _out_edge(state, conv, "Y")
+        if y_e is None or not isinstance(y_e.dst, AccessNode):
+            continue
+        use = _single_consumer(sdfg, state, y_e.dst)
+        if use is None or not _is_op(use.dst, "BatchNormalization") or use.dst_conn != "X":
+            continue
+        bn = use.dst
+        if len(state.out_edges(bn)) != 1 or _out_edge(state, bn, "Y") is None:
+            continue        # training outputs present
+        w = constant(conv, "W")
+        params = [constant(bn, c) for c in ("scale", "B", "mean", "var")]
+        has_bias = _in_edge(state, conv, "B") is not None
+        bias = constant(conv, "B") if has_bias else None
+        if w is None or any(p is None for p in params) or (has_bias and bias is None):
+            continue
+        oc = w[1].shape[0]
+        if any(tuple(p[1].shape) != (oc, ) for p in params) or (bias is not None and tuple(bias[1].shape) != (oc, )):
+            continue
+        eps = 1e-5 if bn.epsilon is None else float(bn.epsilon)
+        scale, beta, mean, var = (p[1].double() for p in params)
+        a = scale / torch.sqrt(var + eps)
+        new_w = (w[1].double() * a.reshape(-1, *([1] * (w[1].dim() - 1)))).float().contiguous()
+        new_b = (((bias[1].double() if bias is not None else torch.zeros_like(mean)) - mean) * a + beta).float().contiguous()
+        w_name, b_name = by_clean[w[0].src.data] + "_bnfold_" + bn.label, by_clean[w[0].src.data] + "_bnfold_bias_" + bn.label
+        model.weights[w_name], model.weights[b_name] = new_w, new_b
+        w_clean, b_clean = clean_onnx_name(w_name), clean_onnx_name(b_name)
+        sdfg.add_array(w_clean, list(new_w.shape), sdfg.arrays[w[0].src.data].dtype, transient=False)
+        sdfg.add_array(b_clean, [oc], sdfg.arrays[w[0].src.data].dtype, transient=False)
+        state.remove_edge(w[0])
+        state.add_edge(state.add_access(w_clean), None, conv, "W", sdfg.make_array_memlet(w_clean))
+        if bias is not None:
+            state.remove_edge(bias[0])
+        else:
+            conv.add_in_connector("B")
+        state.add_edge(state.add_access(b_clean), None, conv, "B", sdfg.make_array_memlet(b_clean))
+        out_e = _out_edge(state, bn, "Y")
+        mid = y_e.dst
+        state.remove_edge(y_e)
+        state.add_edge(conv, "Y", out_e.dst, None, sdfg.make_array_memlet(out_e.dst.data))
+        state.remove_node(bn)
+        state.remove_node(mid)
+        del sdfg.arrays[mid.data]
+        folded += 1
+    return folded
+
+
 def _fold_into_contractions(sdfg: SDFG, state: SDFGState) -> int:
     folded = 0
     changed = True
@@ -1156,6 +1227,7 @@ def fuse_onnx_graph(sdfg: SDFG) -> int:
     total = 0
     for state in sdfg.nodes():
         total += _fuse_pad_conv(sdfg, state)
+        total += _fold_batchnorm_into_conv(sdfg, state)
         total += _fuse_decomposed_layernorm(sdfg, state)
         total += _fuse_decomposed_gelu(sdfg, state)
         total += _fold_into_contractions(sdfg, state)

@@ -432,3 +432,19 @@ def test_reference_bert_subgraph_fixture(fold):
         cast = saved["bertSLASHembeddingsSLASHReshape_4__42COLON0"]
         assert cast.dtype == torch.int64
         assert torch.equal(cast.type(torch.int32).cpu(), model.weights["bert/embeddings/Reshape_4/shape:0"].cpu())
+
+
+@pytest.mark.parametrize("conv_bias", [True, False])
+@pytest.mark.parametrize("fuse", [True, False])
+def test_conv_batchnorm_relu_values(conv_bias, fuse):
+    # Conv -> BatchNormalization -> Relu: folded into one convolution launch, or three launches, against the
+    # oracle's convolution followed by the inference batch normalization
+    from test_fusion import _conv_bn_model
+    m, w, p = _conv_bn_model(conv_bias=conv_bias)
+    x = np.random.default_rng(11).normal(size=(2, 3, 8, 8)).astype(np.float32)
+    model = donnx.ONNXModel(f"conv_bn_values_{conv_bias}_{fuse}", m, fuse=fuse)
+    got = model(x)
+    conv = O.conv2d(x, w, p["cb"] if conv_bias else None, pads=(1, 1, 1, 1))
+    expected = O.relu(O.batch_normalization(conv, p["scale"], p["beta"], p["mean"], p["var"], 1e-3))
+    assert rel_err(expected, got) < FP32_REL_TOL
+    assert model.compile_and_init().num_launches == (1 if fuse else 3)

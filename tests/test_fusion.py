@@ -305,3 +305,48 @@ def test_pad_conv_fusion():
         model = donnx.ONNXModel("pad_kept", _pad_conv_model(**kwargs))
         with pytest.raises(ExpansionRefused, match="Pad"):
             model.expand()
+
+
+def _conv_bn_model(conv_bias=True, second_reader=False, variable_scale=False, relu=True):
+    T = proto.TensorProto
+    rng = np.random.default_rng(7)
+    w = rng.normal(size=(4, 3, 3, 3)).astype(np.float32)
+    params = {"scale": rng.normal(size=4), "beta": rng.normal(size=4), "mean": rng.normal(size=4), "var": rng.uniform(0.5, 2.0, size=4),
+              "cb": rng.normal(size=4)}
+    inits = [proto.numpy_helper.from_array(w, name="w")] + \
+        [proto.numpy_helper.from_array(v.astype(np.float32), name=k) for k, v in params.items() if not (variable_scale and k == "scale")]
+    nodes = [H.make_node("Conv", ["x", "w"] + (["cb"] if conv_bias else []), ["c"], pads=[1, 1, 1, 1]),
+             H.make_node("BatchNormalization", ["c", "scale", "beta", "mean", "var"], ["b"], epsilon=1e-3)]
+    ins = [H.make_tensor_value_info("x", T.FLOAT, [2, 3, 8, 8])]
+    if variable_scale:
+        ins.append(H.make_tensor_value_info("scale", T.FLOAT, [4]))
+    outs = []
+    if relu:
+        nodes.append(H.make_node("Relu", ["b"], ["y"]))
+    if second_reader:
+        nodes.append(H.make_node("Relu", ["c"], ["r"]))
+        outs.append(H.make_tensor_value_info("r", T.FLOAT, None))
+    outs.insert(0, H.make_tensor_value_info("y" if relu else "b", T.FLOAT, [2, 4, 8, 8]))
+    g = H.make_graph(nodes, "g", ins, outs, initializer=inits)
+    return H.make_model(g, opset_imports=[H.make_opsetid("", 12)]), w, {k: v.astype(np.float32) for k, v in params.items()}
+
+
+def test_batchnorm_folds_into_the_convolution():
+    # Conv -> BatchNormalization (inference, constant parameters) -> Relu is one convolution launch with new weights
+    for conv_bias in (True, False):
+        m, w, p = _conv_bn_model(conv_bias=conv_bias)
+        model = donnx.ONNXModel(f"conv_bn_{conv_bias}", m)
+        calls = _launches(model)
+        assert [f for f, _ in calls] == ["mi355x_conv2d_f32"]
+        a = p["scale"].astype(np.float64) / np.sqrt(p["var"].astype(np.float64) + 1e-3)
+        folded_w = [v for k, v in model.weights.items() if "_bnfold_" in k and "bias" not in k][0].cpu().numpy()
+        folded_b = [v for k, v in model.weights.items() if "_bnfold_bias_" in k][0].cpu().numpy()
+        assert np.allclose(folded_w, w * a.reshape(-1, 1, 1, 1), rtol=1e-6)
+        assert np.allclose(folded_b, ((p["cb"] if conv_bias else 0.0) - p["mean"]) * a + p["beta"], rtol=1e-5, atol=1e-6)
+        assert np.array_equal(model.weights["w"].cpu().numpy(), w)          # the original stays as it was
+    # not folded: the convolution's result has another reader, or a parameter is a graph input
+    for kwargs in (dict(second_reader=True), dict(variable_scale=True)):
+        calls = _launches(donnx.ONNXModel("conv_bn_kept", _conv_bn_model(**kwargs)[0]))
+        assert "mi355x_batchnorm_f32" in [f for f, _ in calls]
+    unfused = _launches(donnx.ONNXModel("conv_bn_plain", _conv_bn_model()[0], fuse=False))
+    assert [f for f, _ in unfused] == ["mi355x_conv2d_f32", "mi355x_batchnorm_f32", "mi355x_eltwise_f32"]

@@ -98,6 +98,51 @@ def test_conv_relu_linear_module_and_decorator():
     assert rel_err(ref2.numpy(), net(x.cuda()).cpu().numpy()) < FP32_REL_TOL
 
 
+def _small_resnet_stem():
+    """Conv, BatchNorm, ReLU, MaxPool, Conv (no bias), BatchNorm, ReLU, global average pooling, Linear: the
+    layer types of a ResNet around its 3 x 3 convolutions, in eval() mode with non-trivial statistics."""
+    torch.manual_seed(5)
+    net = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.BatchNorm2d(8), nn.ReLU(), nn.MaxPool2d(3, 2, 1),
+                        nn.Conv2d(8, 16, 3, padding=1, bias=False), nn.BatchNorm2d(16, eps=1e-3), nn.ReLU(),
+                        nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(16, 10)).eval()
+    with torch.no_grad():
+        for m in net:
+            if isinstance(m, nn.BatchNorm2d):
+                m.running_mean.normal_()
+                m.running_var.uniform_(0.5, 2.0)
+                m.weight.normal_()
+                m.bias.normal_()
+    return net
+
+
+@pytest.mark.parametrize("exporter", ["structural", "torch"])
+def test_conv_batchnorm_pool_network_launch_list(exporter):
+    net = _small_resnet_stem()
+    dummy = (torch.randn(2, 3, 16, 16), )
+    dm = DaceModule(net, dummy_inputs=dummy, exporter=exporter)
+    # both BatchNormalizations folded into their convolutions, both ReLUs into the convolutions' epilogues
+    assert _functions(dm) == ["mi355x_conv2d_f32", "mi355x_maxpool2d_f32", "mi355x_conv2d_f32", "mi355x_reduce_mean_f32",
+                              "mi355x_gemm_f32"]
+    plain = DaceModule(net, dummy_inputs=dummy, exporter=exporter, auto_optimize=False)
+    assert sorted(_functions(plain)) == sorted(["mi355x_conv2d_f32", "mi355x_batchnorm_f32", "mi355x_eltwise_f32"] * 2 +
+                                               ["mi355x_maxpool2d_f32", "mi355x_reduce_mean_f32", "mi355x_gemm_f32"])
+    with pytest.raises(UnsupportedModule, match="eval"):
+        module_to_onnx(copy.deepcopy(net).train(), dummy)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("exporter", ["structural", "torch"])
+def test_conv_batchnorm_pool_network_results(exporter):
+    net = _small_resnet_stem()
+    x = torch.randn(4, 3, 16, 16)
+    with torch.no_grad():
+        ref = copy.deepcopy(net).double()(x.double())
+    got = DaceModule(net, exporter=exporter)(x.cuda())
+    assert rel_err(ref.numpy(), got.cpu().numpy()) < FP32_REL_TOL
+    plain = DaceModule(net, exporter=exporter, auto_optimize=False)
+    assert rel_err(ref.numpy(), plain(x.cuda()).cpu().numpy()) < FP32_REL_TOL
+
+
 # ----------------------------------------------------------------------------- the TorchScript exporter path
 class _TwoInputNet(nn.Module):
     """Not a Sequential and with two inputs: only the exporter can turn it into a graph."""
