@@ -143,6 +143,50 @@ def test_conv_batchnorm_pool_network_results(exporter):
     assert rel_err(ref.numpy(), plain(x.cuda()).cpu().numpy()) < FP32_REL_TOL
 
 
+class _ResidualBlock(nn.Module):
+    """A ResNet basic block with a projection shortcut (not a Sequential: only the exporter can write it)."""
+    def __init__(self, c):
+        super().__init__()
+        self.c1, self.b1 = nn.Conv2d(c, c, 3, padding=1, bias=False), nn.BatchNorm2d(c)
+        self.c2, self.b2 = nn.Conv2d(c, c, 3, padding=1, bias=False), nn.BatchNorm2d(c)
+        self.down = nn.Sequential(nn.Conv2d(c, c, 1, bias=False), nn.BatchNorm2d(c))
+
+    def forward(self, x):
+        h = torch.relu(self.b1(self.c1(x)))
+        return torch.relu(self.b2(self.c2(h)) + self.down(x))
+
+
+def _residual_block():
+    torch.manual_seed(6)
+    net = _ResidualBlock(16).eval()
+    with torch.no_grad():
+        for m in net.modules():
+            if isinstance(m, nn.BatchNorm2d):
+                m.running_mean.normal_(std=0.3)
+                m.running_var.uniform_(0.5, 2.0)
+                m.weight.normal_(1.0, 0.2)
+                m.bias.normal_(std=0.2)
+    return net
+
+
+def test_residual_block_launch_list():
+    dm = DaceModule(_residual_block(), dummy_inputs=(torch.randn(2, 16, 8, 8), ))
+    assert [n.op_type for n in dm.onnx_model.graph.node] == ["Conv", "BatchNormalization", "Relu", "Conv", "BatchNormalization",
+                                                             "Conv", "BatchNormalization", "Add", "Relu"]
+    # three convolutions with their normalizations (and the first ReLU) inside, then add + ReLU as one program
+    assert _functions(dm) == ["mi355x_conv2d_f32"] * 3 + ["mi355x_eltwise_program_f32"]
+
+
+@pytest.mark.gpu
+def test_residual_block_results():
+    net = _residual_block()
+    x = torch.randn(3, 16, 8, 8)
+    with torch.no_grad():
+        ref = copy.deepcopy(net).double()(x.double())
+    assert rel_err(ref.numpy(), DaceModule(net)(x.cuda()).cpu().numpy()) < FP32_REL_TOL
+    assert rel_err(ref.numpy(), DaceModule(net, auto_optimize=False)(x.cuda()).cpu().numpy()) < FP32_REL_TOL
+
+
 # ----------------------------------------------------------------------------- the TorchScript exporter path
 class _TwoInputNet(nn.Module):
     """Not a Sequential and with two inputs: only the exporter can turn it into a graph."""
