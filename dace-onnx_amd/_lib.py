@@ -18,7 +18,7 @@ LIBRARY_PATH = os.path.join(_HERE, LIBRARY_NAME)
 
 # status codes / flags, mirrored from include/mi355x_onnx.h
 OK = 0
-EPI_NONE, EPI_BIAS, EPI_RELU, EPI_GELU, EPI_RESIDUAL = 0, 1, 2, 4, 8
+EPI_NONE, EPI_BIAS, EPI_RELU, EPI_GELU, EPI_RESIDUAL, EPI_RELU_AFTER = 0, 1, 2, 4, 8, 16
 OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_POW = 0, 1, 2, 3, 4
 OP_RELU, OP_GELU, OP_ERF, OP_SQRT, OP_COPY = 16, 17, 18, 19, 20
 REDUCE_MEAN, REDUCE_SUM, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
@@ -42,6 +42,8 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
                                _c_i64_p, _c_i64_p, _c_i64_p, _c_i64_p, _f32, _int, _vp]),
     "mi355x_conv2d_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                  _c_i64_p, _c_i64_p, _c_i64_p, _int, _vp]),
+    "mi355x_conv2d_res_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                     _c_i64_p, _c_i64_p, _c_i64_p, _int, _vp]),
     "mi355x_matmul_integer_i8": (_int, [_vp, _vp, _vp, _vp, _vp,
                                         _i64, _i64, _i64, _vp]),
     "mi355x_softmax_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
@@ -49,7 +51,7 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
                                     _c_i64_p, _c_i64_p, _c_i64_p, _c_i64_p, _f32, _vp]),
     "mi355x_layernorm_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "mi355x_reduce_mean_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
-    "mi355x_maxpool2d_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "mi355x_maxpool2d_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _c_i64_p, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_batchnorm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),
     "mi355x_cast": (_int, [_vp, _int, _vp, _int, _i64, _vp]),
     "mi355x_reduce_f32": (_int, [_int, _vp, _vp, _i64, _i64, _i64, _vp]),

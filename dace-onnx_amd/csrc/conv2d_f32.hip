@@ -44,8 +44,22 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv& f) {
     return f.d == 1 ? n : (__umulhi(n, f.mul) >> f.shr);
 }
 
+// The part of the epilogue after bias and activation: the residual (same layout as Y, hence the same
+// offset) and the activation that follows it (the last two steps of a ResNet block).
+__device__ __forceinline__ f32x4 conv_epilogue_tail4(f32x4 v, int epi, const float* residual, int64_t off) {
+    if (epi & MI355X_EPI_RESIDUAL) v += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(residual + off));
+    if (epi & MI355X_EPI_RELU_AFTER) v = f32x4{fmaxf(v.x, 0.f), fmaxf(v.y, 0.f), fmaxf(v.z, 0.f), fmaxf(v.w, 0.f)};
+    return v;
+}
+__device__ __forceinline__ float conv_epilogue_tail1(float v, int epi, const float* residual, int64_t off) {
+    if (epi & MI355X_EPI_RESIDUAL) v += residual[off];
+    if (epi & MI355X_EPI_RELU_AFTER) v = fmaxf(v, 0.f);
+    return v;
+}
+
 struct ConvArgs {
     const float* X; const float* W; const float* bias; float* Y;
+    const float* residual;   // laid out like Y; read only with MI355X_EPI_RESIDUAL
     int N, C, H, Wd, M, KH, KW, OH, OW;
     int pad_t, pad_l, stride_h, stride_w, dil_h, dil_w;
     int K;          // C*KH*KW
@@ -180,15 +194,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv2d_f32_kernel(Conv
                 // OH*OW % 4 == 0: the four positions share an image and are adjacent
                 const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
                 const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
-                float* dst = p.Y + ((int64_t)n * p.M + oc) * p.OHW + q;
-                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst));
+                const int64_t off = ((int64_t)n * p.M + oc) * p.OHW + q;
+                __builtin_nontemporal_store(conv_epilogue_tail4(v, p.epi, p.residual, off), reinterpret_cast<f32x4*>(p.Y + off));
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     if (pp + r >= p.P) break;
                     const uint32_t n = fdiv((uint32_t)(pp + r), p.div_ohw);
                     const uint32_t q = (uint32_t)(pp + r) - n * (uint32_t)p.OHW;
-                    p.Y[((int64_t)n * p.M + oc) * p.OHW + q] = v[r];
+                    const int64_t off = ((int64_t)n * p.M + oc) * p.OHW + q;
+                    p.Y[off] = conv_epilogue_tail1(v[r], p.epi, p.residual, off);
                 }
             }
         }
@@ -427,14 +442,16 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
         if (p.vec_y) {
             const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
             const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
-            __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(p.Y + ((int64_t)n * p.M + oc) * p.OHW + q));
+            const int64_t off = ((int64_t)n * p.M + oc) * p.OHW + q;
+            __builtin_nontemporal_store(conv_epilogue_tail4(v, p.epi, p.residual, off), reinterpret_cast<f32x4*>(p.Y + off));
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 if (pp + r >= p.P) break;
                 const uint32_t n = fdiv((uint32_t)(pp + r), p.div_ohw);
                 const uint32_t q = (uint32_t)(pp + r) - n * (uint32_t)p.OHW;
-                p.Y[((int64_t)n * p.M + oc) * p.OHW + q] = v[r];
+                const int64_t off = ((int64_t)n * p.M + oc) * p.OHW + q;
+                p.Y[off] = conv_epilogue_tail1(v[r], p.epi, p.residual, off);
             }
         }
     }
@@ -473,15 +490,26 @@ extern "C" int mi355x_conv2d_f32(const float* X, const float* W, const float* bi
                                  int64_t KH, int64_t KW, const int64_t* pads,
                                  const int64_t* strides, const int64_t* dilations, int epilogue,
                                  void* stream) {
+    MI355X_REQUIRE((epilogue & ~(MI355X_EPI_BIAS | MI355X_EPI_RELU)) == 0,
+                   "conv2d: epilogue 0x%x not supported (bias and relu only)", epilogue);
+    return mi355x_conv2d_res_f32(X, W, bias, nullptr, Y, N, C, H, Wd, M, KH, KW, pads, strides, dilations, epilogue, stream);
+}
+
+extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float* bias, const float* residual,
+                                     float* Y, int64_t N, int64_t C, int64_t H, int64_t Wd, int64_t M,
+                                     int64_t KH, int64_t KW, const int64_t* pads,
+                                     const int64_t* strides, const int64_t* dilations, int epilogue,
+                                     void* stream) {
     using namespace mi355x;
     MI355X_REQUIRE(N >= 0 && C >= 0 && H >= 0 && Wd >= 0 && M >= 0 && KH >= 1 && KW >= 1,
                    "conv2d: bad extents N=%lld C=%lld H=%lld W=%lld M=%lld KH=%lld KW=%lld",
                    (long long)N, (long long)C, (long long)H, (long long)Wd, (long long)M,
                    (long long)KH, (long long)KW);
     MI355X_REQUIRE(pads && strides && dilations, "conv2d: null pads/strides/dilations");
-    MI355X_REQUIRE((epilogue & ~(MI355X_EPI_BIAS | MI355X_EPI_RELU)) == 0,
-                   "conv2d: epilogue 0x%x not supported (bias and relu only)", epilogue);
+    MI355X_REQUIRE((epilogue & ~(MI355X_EPI_BIAS | MI355X_EPI_RELU | MI355X_EPI_RESIDUAL | MI355X_EPI_RELU_AFTER)) == 0,
+                   "conv2d: epilogue 0x%x not supported (bias, relu, residual, relu after the residual)", epilogue);
     MI355X_REQUIRE(!(epilogue & MI355X_EPI_BIAS) || bias, "conv2d: MI355X_EPI_BIAS without bias");
+    MI355X_REQUIRE(!(epilogue & MI355X_EPI_RESIDUAL) || residual, "conv2d: MI355X_EPI_RESIDUAL without residual");
     for (int i = 0; i < 4; ++i) MI355X_REQUIRE(pads[i] >= 0, "conv2d: negative pad");
     for (int i = 0; i < 2; ++i)
         MI355X_REQUIRE(strides[i] >= 1 && dilations[i] >= 1, "conv2d: stride/dilation must be >= 1");
@@ -497,7 +525,7 @@ extern "C" int mi355x_conv2d_f32(const float* X, const float* W, const float* bi
                    "conv2d: tensor too large for 32-bit gather offsets");
 
     ConvArgs p;
-    p.X = X; p.W = W; p.bias = bias; p.Y = Y;
+    p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.residual = residual;
     p.N = (int)N; p.C = (int)C; p.H = (int)H; p.Wd = (int)Wd; p.M = (int)M; p.KH = (int)KH; p.KW = (int)KW;
     p.OH = (int)OH; p.OW = (int)OW; p.OHW = (int)(OH * OW);
     p.pad_t = (int)pads[0]; p.pad_l = (int)pads[1];
@@ -509,7 +537,7 @@ extern "C" int mi355x_conv2d_f32(const float* X, const float* W, const float* bi
     p.epi = epilogue;
     auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     p.vec_w = (K % 4 == 0) && al16(W);
-    p.vec_y = ((OH * OW) % 4 == 0) && al16(Y);
+    p.vec_y = ((OH * OW) % 4 == 0) && al16(Y) && (!(epilogue & MI355X_EPI_RESIDUAL) || al16(residual));
 
     int cus = mi355x_device_cu_count();
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "conv2d: no usable HIP device");

@@ -408,8 +408,9 @@ def _conv_geometry(node, X, W):
 @op_implementation(op="Conv", name=IMPLEMENTATION_NAME)
 class MI355XConv(ONNXForward):
     """2-D NCHW convolution as implicit GEMM on MFMA. Honours ``strides``,
-    ``pads`` (also asymmetric), ``dilations`` and ``auto_pad``; the bias and a
-    following Relu are applied in the kernel's epilogue. PureConv2D refuses any
+    ``pads`` (also asymmetric), ``dilations`` and ``auto_pad``; the bias, a
+    following Relu, a residual Add and the Relu after it (attached by the fusion pass as ``_activation``,
+    ``_residual``, ``_activation_after``) are applied in the kernel's epilogue. PureConv2D refuses any
     non-zero pad and ignores the stride (img_op_implementations.py:201-203,278)."""
 
     @staticmethod
@@ -433,20 +434,30 @@ class MI355XConv(ONNXForward):
             return False
         if prod(X.shape) >= 2**30 or prod(Y.shape) >= 2**31:
             return False
-        return True
+        if _has_input(node, state, "_residual"):     # attached by the fusion pass: a tensor exactly like Y
+            R = in_desc_with_name(node, state, sdfg, "_residual")
+            if not _is_f32(R) or not _contig(R) or tuple(R.shape) != tuple(Y.shape):
+                return False
+        elif getattr(node, "_activation_after", None):
+            return False
+        return getattr(node, "_activation", None) in (None, "relu") and getattr(node, "_activation_after", None) in (None, "relu")
 
     @staticmethod
     def forward(node, state: SDFGState, sdfg: SDFG):
         X = in_desc_with_name(node, state, sdfg, "X")
         W = in_desc_with_name(node, state, sdfg, "W")
-        has_bias = _has_input(node, state, "B")
+        has_bias, has_res = _has_input(node, state, "B"), _has_input(node, state, "_residual")
         pads, strides, dil, _, _ = _conv_geometry(node, X, W)
         epi = (_lib.EPI_BIAS if has_bias else 0) | (_lib.EPI_RELU if getattr(node, "_activation", None) == "relu" else 0)
         N, C, H, Wd = X.shape
         M, _, KH, KW = W.shape
-        return kernel_call_for_node(node, state, "mi355x_conv2d_f32", [
-            Ptr("X"), Ptr("W"), Ptr("B" if has_bias else None), Ptr("Y"),
-            N, C, H, Wd, M, KH, KW, I64Array(pads), I64Array(strides), I64Array(dil), epi, Stream()])
+        geometry = [N, C, H, Wd, M, KH, KW, I64Array(pads), I64Array(strides), I64Array(dil)]
+        if not has_res:
+            return kernel_call_for_node(node, state, "mi355x_conv2d_f32", [
+                Ptr("X"), Ptr("W"), Ptr("B" if has_bias else None), Ptr("Y")] + geometry + [epi, Stream()])
+        epi |= _lib.EPI_RESIDUAL | (_lib.EPI_RELU_AFTER if getattr(node, "_activation_after", None) == "relu" else 0)
+        return kernel_call_for_node(node, state, "mi355x_conv2d_res_f32", [
+            Ptr("X"), Ptr("W"), Ptr("B" if has_bias else None), Ptr("_residual"), Ptr("Y")] + geometry + [epi, Stream()])
 
 
 @op_implementation(op="MaxPool", name=IMPLEMENTATION_NAME)

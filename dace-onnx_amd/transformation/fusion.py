@@ -323,8 +323,15 @@ def _fold_into_contractions(sdfg: SDFG, state: SDFGState) -> int:
                     folded += 1
                     changed = True
                     break
-            # ---- residual (last in the epilogue)
-            if _is_op(node, "MatMul") and _is_op(nxt, "Add") and not has_res:
+            # ---- convolution: the Relu after the residual (the end of a ResNet block)
+            if _is_op(node, "Conv") and has_res and _is_op(nxt, "Relu") and getattr(node, "_activation_after", None) is None:
+                node._activation_after = "relu"
+                _replace_output(sdfg, state, node, "Y", nxt, "Y")
+                folded += 1
+                changed = True
+                break
+            # ---- residual (after bias and activation in the epilogue)
+            if _is_op(node, "MatMul", "Conv") and _is_op(nxt, "Add") and not has_res:
                 other_conn = "B" if use.dst_conn == "A" else "A"
                 other = _in_edge(state, nxt, other_conn)
                 if other is not None:

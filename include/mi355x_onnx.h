@@ -65,6 +65,8 @@ int mi355x_device_cu_count(void);
 #define MI355X_EPI_RELU 2
 #define MI355X_EPI_GELU 4
 #define MI355X_EPI_RESIDUAL 8
+/* convolution only: v = max(v, 0) once more after the residual (the end of a ResNet block) */
+#define MI355X_EPI_RELU_AFTER 16
 
 /* ONNX MatMul / Gemm, fp32, on MFMA.
  *   C[b0,b1,m,n] = epilogue(alpha * sum_k A[b0,b1,m,k] * B[b0,b1,k,n])
@@ -103,6 +105,16 @@ int mi355x_conv2d_f32(const float* X, const float* W, const float* bias, float* 
                       int64_t M, int64_t KH, int64_t KW,
                       const int64_t* pads, const int64_t* strides,
                       const int64_t* dilations, int epilogue, void* stream);
+
+/* The same convolution with a residual: `residual` has the shape and layout of Y and is added after
+ * bias and activation (MI355X_EPI_RESIDUAL); MI355X_EPI_RELU_AFTER applies max(v, 0) to the sum. Stands
+ * for Conv -> Add -> Relu, three nodes (and two more passes over the result) in the reference's graphs
+ * (img_op_implementations.py:164-326, pure_implementations.py:77-79, 462-474). */
+int mi355x_conv2d_res_f32(const float* X, const float* W, const float* bias, const float* residual,
+                          float* Y, int64_t N, int64_t C, int64_t H, int64_t Wd,
+                          int64_t M, int64_t KH, int64_t KW,
+                          const int64_t* pads, const int64_t* strides,
+                          const int64_t* dilations, int epilogue, void* stream);
 
 /* ONNX MaxPool, 2-D, fp32, NCHW: Y[n,c,oh,ow] = max over the KH x KW window at
  * (oh * strides[0] - pads[0] + kh * dilations[0], ow * strides[1] - pads[1] + kw * dilations[1]);

@@ -448,3 +448,35 @@ def test_conv_batchnorm_relu_values(conv_bias, fuse):
     expected = O.relu(O.batch_normalization(conv, p["scale"], p["beta"], p["mean"], p["var"], 1e-3))
     assert rel_err(expected, got) < FP32_REL_TOL
     assert model.compile_and_init().num_launches == (1 if fuse else 3)
+
+
+@pytest.mark.parametrize("shape, wshape, pads, strides", [
+    ((4, 64, 28, 28), (64, 64, 3, 3), [1, 1, 1, 1], [1, 1]),      # K % 32 == 0: the gather kernel, 16-byte stores
+    ((2, 32, 15, 15), (48, 32, 3, 3), [1, 1, 1, 1], [2, 2]),      # 8 x 8 output
+    ((3, 3, 9, 11), (5, 3, 3, 3), [0, 1, 2, 0], [1, 1]),          # generic kernel, OH * OW odd: scalar stores
+    ((2, 16, 8, 8), (16, 16, 1, 1), [0, 0, 0, 0], [1, 1])])       # 1 x 1 projection shortcut
+@pytest.mark.parametrize("epi", [_lib.EPI_RESIDUAL, _lib.EPI_BIAS | _lib.EPI_RESIDUAL | _lib.EPI_RELU_AFTER,
+                                 _lib.EPI_BIAS | _lib.EPI_RELU | _lib.EPI_RESIDUAL | _lib.EPI_RELU_AFTER])
+def test_conv_residual_epilogue(shape, wshape, pads, strides, epi):
+    """relu?(relu?(conv + bias) + residual) in the convolution's epilogue against the oracle's Conv, Add, Relu."""
+    rng = np.random.default_rng(12)
+    x = rng.normal(size=shape).astype(np.float32)
+    w = (rng.normal(size=wshape) / np.sqrt(np.prod(wshape[1:]))).astype(np.float32)
+    b = rng.normal(size=wshape[0]).astype(np.float32)
+    pre = O.conv2d(x, w, b if epi & _lib.EPI_BIAS else None, strides=tuple(strides), pads=tuple(pads))
+    r = rng.normal(size=pre.shape).astype(np.float32)
+    expected = (O.relu(pre) if epi & _lib.EPI_RELU else pre) + r
+    expected = O.relu(expected) if epi & _lib.EPI_RELU_AFTER else expected
+    tx, tw, tb, tr = (torch.from_numpy(a).cuda() for a in (x, w, b, r))
+    y = torch.full(pre.shape, float("nan"), device="cuda")
+    lib = _lib.library()
+    args = [tx.data_ptr(), tw.data_ptr(), tb.data_ptr() if epi & _lib.EPI_BIAS else None, tr.data_ptr(), y.data_ptr(),
+            *shape, wshape[0], wshape[2], wshape[3], _lib.i64_array(pads), _lib.i64_array(strides), _lib.i64_array([1, 1]),
+            epi, torch.cuda.current_stream().cuda_stream]
+    assert lib.mi355x_conv2d_res_f32(*args) == 0, lib.mi355x_last_error()
+    torch.cuda.synchronize()
+    assert rel_err(expected, y.cpu().numpy()) < FP32_REL_TOL
+    # the flags are checked: a residual flag without a residual, or an unknown flag, launches nothing
+    args[3] = None
+    assert lib.mi355x_conv2d_res_f32(*args) == 1 and b"without residual" in lib.mi355x_last_error()
+    assert lib.mi355x_conv2d_f32(*(args[:3] + args[4:-2] + [_lib.EPI_RESIDUAL, None])) == 1

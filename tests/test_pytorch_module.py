@@ -173,8 +173,12 @@ def test_residual_block_launch_list():
     dm = DaceModule(_residual_block(), dummy_inputs=(torch.randn(2, 16, 8, 8), ))
     assert [n.op_type for n in dm.onnx_model.graph.node] == ["Conv", "BatchNormalization", "Relu", "Conv", "BatchNormalization",
                                                              "Conv", "BatchNormalization", "Add", "Relu"]
-    # three convolutions with their normalizations (and the first ReLU) inside, then add + ReLU as one program
-    assert _functions(dm) == ["mi355x_conv2d_f32"] * 3 + ["mi355x_eltwise_program_f32"]
+    # three convolutions with their normalizations inside; the first takes its ReLU, the last to run takes the
+    # other branch as its residual and the ReLU after the sum (bias | residual | relu-after = 25)
+    calls = [n for n, _ in dm.dace_model.expand().all_nodes_recursive() if isinstance(n, dace.KernelCall)]
+    assert sorted(c.function for c in calls) == ["mi355x_conv2d_f32"] * 2 + ["mi355x_conv2d_res_f32"]
+    assert [c.args[-2] for c in calls if c.function == "mi355x_conv2d_res_f32"] == [25]
+    assert sorted(c.args[-2] for c in calls if c.function == "mi355x_conv2d_f32") == [1, 3]
 
 
 @pytest.mark.gpu
@@ -227,7 +231,8 @@ def test_auto_falls_back_to_the_exporter():
         DaceModule(net, dummy_inputs=(torch.randn(2, 3, 8, 8), torch.randn(2, 8, 8, 8)), exporter="structural")
     dm = DaceModule(net, dummy_inputs=(torch.randn(2, 3, 8, 8), torch.randn(2, 8, 8, 8)))
     assert len(dm.dace_model.inputs) == 2
-    assert _functions(dm) == ["mi355x_conv2d_f32", "mi355x_eltwise_f32", "mi355x_gemm_f32", "mi355x_softmax_f32"]
+    # relu(conv(x)) + y: ReLU and the second input both ride in the convolution's epilogue
+    assert _functions(dm) == ["mi355x_conv2d_res_f32", "mi355x_gemm_f32", "mi355x_softmax_f32"]
 
 
 @pytest.mark.gpu
