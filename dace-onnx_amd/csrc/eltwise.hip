@@ -139,13 +139,30 @@ __global__ __launch_bounds__(256) void permute_tiled(const uint32_t* __restrict_
     }
 }
 
-// ONNX Cast: Y[i] = (TO)X[i]; to bool is X[i] != 0 (stored as one byte).
+// ONNX Cast: Y[i] = (TO)X[i]; to bool is X[i] != 0 (stored as one byte). VEC: four elements per lane and
+// access (both pointers aligned to four elements), the last n % 4 elements one by one.
+template <class T> using Vec4 = T __attribute__((ext_vector_type(4)));
+
 template <class FROM, class TO, bool TO_BOOL>
+__device__ __forceinline__ TO cast_one(FROM v) {
+    if constexpr (TO_BOOL) return (TO)(v != (FROM)0);
+    else return (TO)v;
+}
+
+template <class FROM, class TO, bool TO_BOOL, bool VEC>
 __global__ __launch_bounds__(256) void cast_kernel(const FROM* __restrict__ X, TO* __restrict__ Y, int64_t n) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-        if constexpr (TO_BOOL) Y[i] = (TO)(X[i] != (FROM)0);
-        else Y[i] = (TO)X[i];
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x, first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if constexpr (VEC) {
+        const Vec4<FROM>* x4 = reinterpret_cast<const Vec4<FROM>*>(X);
+        Vec4<TO>* y4 = reinterpret_cast<Vec4<TO>*>(Y);
+        for (int64_t i = first; i < n / 4; i += stride) {
+            const Vec4<FROM> v = x4[i];
+            y4[i] = Vec4<TO>{cast_one<FROM, TO, TO_BOOL>(v.x), cast_one<FROM, TO, TO_BOOL>(v.y),
+                             cast_one<FROM, TO, TO_BOOL>(v.z), cast_one<FROM, TO, TO_BOOL>(v.w)};
+        }
+        for (int64_t i = (n / 4) * 4 + first; i < n; i += stride) Y[i] = cast_one<FROM, TO, TO_BOOL>(X[i]);
+    } else {
+        for (int64_t i = first; i < n; i += stride) Y[i] = cast_one<FROM, TO, TO_BOOL>(X[i]);
     }
 }
 
@@ -260,18 +277,25 @@ extern "C" int mi355x_eltwise_f32(int op, const float* A, const float* B, float*
 
 namespace mi355x {
 
+template <class FROM, class TO, bool TO_BOOL>
+static void launch_cast_to(const void* X, void* Y, int64_t n, hipStream_t st) {
+    const FROM* x = static_cast<const FROM*>(X);
+    TO* y = static_cast<TO*>(Y);
+    const bool vec = reinterpret_cast<uintptr_t>(X) % (4 * sizeof(FROM)) == 0 && reinterpret_cast<uintptr_t>(Y) % (4 * sizeof(TO)) == 0 && n >= 4;
+    if (vec) hipLaunchKernelGGL((cast_kernel<FROM, TO, TO_BOOL, true>), dim3(grid_for(n / 4)), dim3(256), 0, st, x, y, n);
+    else hipLaunchKernelGGL((cast_kernel<FROM, TO, TO_BOOL, false>), dim3(grid_for(n)), dim3(256), 0, st, x, y, n);
+}
+
 template <class FROM>
 static int launch_cast_from(const void* X, void* Y, int to_type, int64_t n, hipStream_t st) {
-    const FROM* x = static_cast<const FROM*>(X);
-    const dim3 grid(grid_for(n)), block(256);
     switch (to_type) {
-        case MI355X_TYPE_FLOAT: hipLaunchKernelGGL((cast_kernel<FROM, float, false>), grid, block, 0, st, x, static_cast<float*>(Y), n); break;
-        case MI355X_TYPE_DOUBLE: hipLaunchKernelGGL((cast_kernel<FROM, double, false>), grid, block, 0, st, x, static_cast<double*>(Y), n); break;
-        case MI355X_TYPE_INT32: hipLaunchKernelGGL((cast_kernel<FROM, int32_t, false>), grid, block, 0, st, x, static_cast<int32_t*>(Y), n); break;
-        case MI355X_TYPE_INT64: hipLaunchKernelGGL((cast_kernel<FROM, int64_t, false>), grid, block, 0, st, x, static_cast<int64_t*>(Y), n); break;
-        case MI355X_TYPE_INT8: hipLaunchKernelGGL((cast_kernel<FROM, int8_t, false>), grid, block, 0, st, x, static_cast<int8_t*>(Y), n); break;
-        case MI355X_TYPE_UINT8: hipLaunchKernelGGL((cast_kernel<FROM, uint8_t, false>), grid, block, 0, st, x, static_cast<uint8_t*>(Y), n); break;
-        case MI355X_TYPE_BOOL: hipLaunchKernelGGL((cast_kernel<FROM, uint8_t, true>), grid, block, 0, st, x, static_cast<uint8_t*>(Y), n); break;
+        case MI355X_TYPE_FLOAT: launch_cast_to<FROM, float, false>(X, Y, n, st); break;
+        case MI355X_TYPE_DOUBLE: launch_cast_to<FROM, double, false>(X, Y, n, st); break;
+        case MI355X_TYPE_INT32: launch_cast_to<FROM, int32_t, false>(X, Y, n, st); break;
+        case MI355X_TYPE_INT64: launch_cast_to<FROM, int64_t, false>(X, Y, n, st); break;
+        case MI355X_TYPE_INT8: launch_cast_to<FROM, int8_t, false>(X, Y, n, st); break;
+        case MI355X_TYPE_UINT8: launch_cast_to<FROM, uint8_t, false>(X, Y, n, st); break;
+        case MI355X_TYPE_BOOL: launch_cast_to<FROM, uint8_t, true>(X, Y, n, st); break;
         default: return set_error(MI355X_ERR_INVALID_ARGUMENT, "cast: unsupported target type %d", to_type);
     }
     return check_launch("cast");

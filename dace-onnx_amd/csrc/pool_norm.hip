@@ -18,8 +18,11 @@ struct PoolArgs {
     int H, W, OH, OW, KH, KW, pad_t, pad_l, sh, sw, dh, dw;
 };
 
+// IEEE-754-2019 maximum: a NaN in either operand gives NaN (numpy's max does the same); one v_maximum3_f32.
+__device__ __forceinline__ float max_nan(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+
 // One thread per output element, adjacent lanes adjacent along OW. Padded positions do not take part in the
-// maximum (ONNX MaxPool pads with -inf); NaN propagates like numpy's max.
+// maximum (ONNX MaxPool pads with -inf).
 __global__ __launch_bounds__(256) void maxpool2d_kernel(PoolArgs p) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < p.total; i += stride) {
@@ -29,19 +32,77 @@ __global__ __launch_bounds__(256) void maxpool2d_kernel(PoolArgs p) {
         const int64_t plane = t / p.OH;                      // n * C + c
         const float* x = p.X + plane * p.H * p.W;
         float m = -INFINITY;
-        bool nan = false;
         for (int kh = 0; kh < p.KH; ++kh) {
             const int ih = oh * p.sh - p.pad_t + kh * p.dh;
             if (ih < 0 || ih >= p.H) continue;
             for (int kw = 0; kw < p.KW; ++kw) {
                 const int iw = ow * p.sw - p.pad_l + kw * p.dw;
                 if (iw < 0 || iw >= p.W) continue;
-                const float v = x[(int64_t)ih * p.W + iw];
-                nan |= v != v;
-                m = fmaxf(m, v);
+                m = max_nan(m, x[(int64_t)ih * p.W + iw]);
             }
         }
-        p.Y[i] = nan ? NAN : m;
+        p.Y[i] = m;
+    }
+}
+
+// The same pooling with the input staged through LDS: a workgroup owns `band` consecutive output rows of one
+// (n, c) plane. The input rows they need are one contiguous piece of the plane, so it is fetched with fully
+// coalesced loads (16 bytes per lane when the piece is aligned) and every element crosses HBM / L2 once, instead of
+// once per window that covers it with stride-`sw` accesses; the band's outputs are one contiguous piece of Y.
+// KH_ / KW_: window extents known at compile time (0: taken from the arguments). A thread walks outputs
+// tid, tid + 256, ... of the band; (oh, ow) advance by (step_oh, step_ow) = divmod(256, OW) without dividing.
+// Windows that lie inside the image -- all but the border -- skip the bounds checks.
+template <bool VEC, int KH_, int KW_>
+__global__ __launch_bounds__(256) void maxpool2d_lds_kernel(PoolArgs p, int band, int bands_per_plane, int step_oh, int step_ow) {
+    extern __shared__ __attribute__((aligned(16))) float rows[];
+    const int KH = KH_ ? KH_ : p.KH, KW = KW_ ? KW_ : p.KW;
+    const int64_t plane = blockIdx.x / bands_per_plane;
+    const int oh0 = (int)(blockIdx.x % bands_per_plane) * band;
+    const int n_oh = min(band, p.OH - oh0);
+    // input rows [ih_lo, ih_hi) of the plane cover every window of the band
+    const int ih_lo = max(oh0 * p.sh - p.pad_t, 0);
+    const int ih_hi = min((oh0 + n_oh - 1) * p.sh - p.pad_t + (KH - 1) * p.dh + 1, p.H);
+    const float* x = p.X + (plane * p.H + ih_lo) * p.W;
+    const int count = (ih_hi - ih_lo) * p.W;
+    if constexpr (VEC) {      // count % 4 == 0 and x 16-byte aligned (checked on the host for every band)
+        const f32x4* x4 = reinterpret_cast<const f32x4*>(x);
+        f32x4* r4 = reinterpret_cast<f32x4*>(rows);
+        for (int i = threadIdx.x; i < count / 4; i += 256) r4[i] = __builtin_nontemporal_load(x4 + i);
+    } else {
+        for (int i = threadIdx.x; i < count; i += 256) rows[i] = x[i];
+    }
+    __syncthreads();
+    float* y = p.Y + (plane * p.OH + oh0) * p.OW;
+    const int eh = (KH - 1) * p.dh + 1, ew = (KW - 1) * p.dw + 1;
+    int oh = oh0 + (int)threadIdx.x / p.OW, ow = (int)threadIdx.x % p.OW;
+    for (int i = threadIdx.x; i < n_oh * p.OW; i += 256) {
+        const int ih0 = oh * p.sh - p.pad_t, iw0 = ow * p.sw - p.pad_l;
+        float m = -INFINITY;
+        if (ih0 >= 0 && ih0 + eh <= p.H && iw0 >= 0 && iw0 + ew <= p.W) {
+            const float* win = rows + (ih0 - ih_lo) * p.W + iw0;
+            if constexpr (KH_ != 0) {
+#pragma unroll
+                for (int kh = 0; kh < KH_; ++kh)
+#pragma unroll
+                    for (int kw = 0; kw < KW_; ++kw) m = max_nan(m, win[kh * p.dh * p.W + kw * p.dw]);
+            } else {
+                for (int kh = 0; kh < KH; ++kh)
+                    for (int kw = 0; kw < KW; ++kw) m = max_nan(m, win[kh * p.dh * p.W + kw * p.dw]);
+            }
+        } else {
+            for (int kh = 0; kh < KH; ++kh) {
+                const int ih = ih0 + kh * p.dh;
+                if (ih < 0 || ih >= p.H) continue;
+                for (int kw = 0; kw < KW; ++kw) {
+                    const int iw = iw0 + kw * p.dw;
+                    if (iw >= 0 && iw < p.W) m = max_nan(m, rows[(ih - ih_lo) * p.W + iw]);
+                }
+            }
+        }
+        y[i] = m;
+        ow += step_ow;
+        oh += step_oh;
+        if (ow >= p.OW) { ow -= p.OW; ++oh; }
     }
 }
 
@@ -97,9 +158,35 @@ extern "C" int mi355x_maxpool2d_f32(const float* X, float* Y, int64_t N, int64_t
     p.H = (int)H; p.W = (int)W; p.OH = (int)OH; p.OW = (int)OW; p.KH = (int)KH; p.KW = (int)KW;
     p.pad_t = (int)pads[0]; p.pad_l = (int)pads[1]; p.sh = (int)strides[0]; p.sw = (int)strides[1];
     p.dh = (int)dilations[0]; p.dw = (int)dilations[1];
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // Staged variant: bands of output rows whose input rows fit 32 KB of LDS and hold about 1024 outputs
+    // (four per thread); planes too wide for that, and launches too small to fill the machine in bands, go direct.
+    constexpr int64_t LDS_FLOATS = 8192;
+    int64_t band = ceil_div((int64_t)1024, OW);
+    band = band < OH ? band : OH;
+    auto rows_needed = [&](int64_t b) { return (b - 1) * strides[0] + eh; };
+    while (band > 1 && rows_needed(band) * W > LDS_FLOATS) --band;
+    const int64_t bands_per_plane = ceil_div(OH, band);
+    const int64_t nwg = N * C * bands_per_plane;
+    if (rows_needed(band) * W <= LDS_FLOATS && nwg < ((int64_t)1 << 31) && total >= 65536) {
+        // 16-byte loads need every band's first input row at a 16-byte boundary: that holds when X is aligned
+        // and W is a multiple of 4 (then any row offset is)
+        const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0;
+        const size_t lds = (size_t)(rows_needed(band) < H ? rows_needed(band) : H) * W * sizeof(float);
+        const dim3 grid((unsigned)nwg), block(256);
+        const int b = (int)band, bpp = (int)bands_per_plane, q = (int)(256 / OW), r = (int)(256 % OW);
+        const int shape = KH == 3 && KW == 3 ? 3 : KH == 2 && KW == 2 ? 2 : 0;
+        if (vec && shape == 3) hipLaunchKernelGGL((maxpool2d_lds_kernel<true, 3, 3>), grid, block, lds, st, p, b, bpp, q, r);
+        else if (vec && shape == 2) hipLaunchKernelGGL((maxpool2d_lds_kernel<true, 2, 2>), grid, block, lds, st, p, b, bpp, q, r);
+        else if (vec) hipLaunchKernelGGL((maxpool2d_lds_kernel<true, 0, 0>), grid, block, lds, st, p, b, bpp, q, r);
+        else if (shape == 3) hipLaunchKernelGGL((maxpool2d_lds_kernel<false, 3, 3>), grid, block, lds, st, p, b, bpp, q, r);
+        else if (shape == 2) hipLaunchKernelGGL((maxpool2d_lds_kernel<false, 2, 2>), grid, block, lds, st, p, b, bpp, q, r);
+        else hipLaunchKernelGGL((maxpool2d_lds_kernel<false, 0, 0>), grid, block, lds, st, p, b, bpp, q, r);
+        return check_launch("maxpool2d_lds_kernel");
+    }
     int64_t blocks = ceil_div(total, (int64_t)256);
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(maxpool2d_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    hipLaunchKernelGGL(maxpool2d_kernel, dim3((unsigned)blocks), dim3(256), 0, st, p);
     return check_launch("maxpool2d_kernel");
 }
 

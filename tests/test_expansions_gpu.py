@@ -474,7 +474,11 @@ def test_einsum_refuses_what_one_gemm_cannot_do(equation, shapes):
     ((5, 3, 10, 10), (2, 2), (2, 2), None, None),                       # LeNet-style pooling
     ((2, 64, 112, 112), (3, 3), (2, 2), (1, 1, 1, 1), None),             # ResNet stem
     ((1, 2, 9, 11), (3, 2), (1, 2), (1, 0, 2, 1), None), ((3, 4, 17, 13), (2, 3), (1, 1), (0, 1, 0, 1), (2, 2)),
-    ((2, 3, 7, 7), (7, 7), None, None, None)])
+    ((2, 3, 7, 7), (7, 7), None, None, None),
+    # large enough for the variant that stages bands of rows through LDS: rows that are not a multiple of 16 bytes,
+    # a window with different extents and dilation, 2 x 2 / 2, and a plane too wide for the staging buffer
+    ((3, 40, 61, 47), (3, 2), (2, 1), (1, 0, 2, 1), (1, 2)), ((2, 48, 56, 56), (2, 2), (2, 2), None, None),
+    ((4, 30, 33, 36), (3, 3), (1, 1), (1, 1, 1, 1), None), ((1, 6, 20, 3000), (3, 3), (2, 2), (1, 1, 1, 1), None)])
 def test_maxpool(shape, kernel, strides, pads, dil):
     """PureMaxPool2D (img_op_implementations.py:28-161), plus pads / dilations: exact."""
     X = np.random.default_rng(27).normal(size=shape).astype(np.float32)
