@@ -67,7 +67,9 @@ class ONNXModel:
                  parent_pytorch_module: typing.Optional[torch.nn.Module] = None,
                  fuse: bool = True,
                  use_hip_graph: bool = False,
-                 save_transients: typing.Optional[typing.Dict[str, torch.Tensor]] = None):
+                 save_transients: typing.Optional[typing.Dict[str, torch.Tensor]] = None,
+                 storage=None,
+                 auto_merge: bool = False):
         """
         :param name: the name for the SDFG.
         :param model: the model to import.
@@ -81,6 +83,9 @@ class ONNXModel:
                                       module are taken from it rather than from the ONNX graph.
         :param fuse: with ``auto_optimize``, fold bias/activation/residual/transposes into contractions.
         :param use_hip_graph: replay the launch sequence as one HIP graph from the second call on.
+        :param storage: kept for signature compatibility (``onnx_importer.py:104``): parameters, inputs and
+                        outputs always live in GPU global memory; anything else named here is an error.
+        :param auto_merge: kept for signature compatibility (symbolic shape merging; shapes are static here).
         :param save_transients: if not None, every intermediate value of the graph is kept and stored in
                                 this dict under its array name on each call (for debugging; as in the
                                 reference, ``onnx_importer.py:454-478``, the intermediates stop being
@@ -88,6 +93,8 @@ class ONNXModel:
         """
         if not isinstance(model, ModelProto):
             model = proto.load(model)
+        if storage is not None and "GPU" not in str(storage):
+            raise ValueError(f"storage {storage!r}: this runner keeps every array in GPU global memory")
         for opset in model.opset_import:
             if opset.domain == "" and opset.version not in (12, 17, 20):
                 log.warning(f"Expected the onnx model to be exported with opset 12, got {opset.version}. "
