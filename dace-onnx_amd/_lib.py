@@ -55,6 +55,7 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
     "mi355x_batchnorm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),
     "mi355x_cast": (_int, [_vp, _int, _vp, _int, _i64, _vp]),
     "mi355x_reduce_f32": (_int, [_int, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "mi355x_reduce_nd_f32": (_int, [_int, _vp, _vp, _int, _c_i64_p, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_log_softmax_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),
     "mi355x_eltwise_f32": (_int, [_int, _vp, _vp, _vp, _int, _c_i64_p, _c_i64_p, _c_i64_p, _vp]),
     "mi355x_permute_b32": (_int, [_vp, _vp, _int, _c_i64_p, _c_i64_p, _vp]),

@@ -93,6 +93,39 @@ __global__ __launch_bounds__(256) void reduce_strided(const float* __restrict__ 
     Y[idx] = R::finish(all, axis_len);
 }
 
+// Reduced axes that are not adjacent (ReduceSum over axes 0 and 2 of [2, 4, 10]): one wave per output element.
+// The kept and the reduced axes are given separately, each with its extents and element strides in X; a lane
+// walks the reduced index space with stride 64 and decomposes its index over the reduced axes.
+struct ReduceNdArgs {
+    int n_keep, n_red;
+    int64_t keep_shape[8], keep_strides[8], red_shape[8], red_strides[8];
+    int64_t n_out, n_red_total;
+};
+
+template <int KIND>
+__global__ __launch_bounds__(256) void reduce_nd(const float* __restrict__ X, float* __restrict__ Y, ReduceNdArgs p) {
+    using R = Reducer<KIND, float>;
+    const int lane = threadIdx.x % WAVE;
+    const int64_t out = (int64_t)blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;
+    if (out >= p.n_out) return;  // whole wave
+    int64_t rem = out, base = 0;
+    for (int d = p.n_keep - 1; d >= 0; --d) {
+        base += (rem % p.keep_shape[d]) * p.keep_strides[d];
+        rem /= p.keep_shape[d];
+    }
+    float s = R::identity();
+    for (int64_t r = lane; r < p.n_red_total; r += WAVE) {
+        int64_t q = r, off = base;
+        for (int d = p.n_red - 1; d >= 0; --d) {
+            off += (q % p.red_shape[d]) * p.red_strides[d];
+            q /= p.red_shape[d];
+        }
+        s = R::combine(s, X[off]);
+    }
+    s = wave_combine<KIND>(s);
+    if (lane == 0) Y[out] = KIND == MI355X_REDUCE_MEAN ? s / (float)p.n_red_total : s;
+}
+
 template <int KIND>
 static int launch_reduce(const float* X, float* Y, int64_t outer, int64_t axis_len, int64_t inner, hipStream_t st) {
     if (inner == 1) {
@@ -132,4 +165,36 @@ extern "C" int mi355x_reduce_f32(int kind, const float* X, float* Y, int64_t out
 extern "C" int mi355x_reduce_mean_f32(const float* X, float* Y, int64_t outer, int64_t axis_len,
                                       int64_t inner, void* stream) {
     return mi355x_reduce_f32(MI355X_REDUCE_MEAN, X, Y, outer, axis_len, inner, stream);
+}
+
+extern "C" int mi355x_reduce_nd_f32(int kind, const float* X, float* Y, int ndim, const int64_t* shape,
+                                    const int64_t* x_strides, const int64_t* reduced, void* stream) {
+    using namespace mi355x;
+    MI355X_REQUIRE(kind >= MI355X_REDUCE_MEAN && kind <= MI355X_REDUCE_MIN, "reduce_nd: unknown kind %d", kind);
+    MI355X_REQUIRE(ndim >= 1 && ndim <= 8 && shape && x_strides && reduced, "reduce_nd: ndim %d outside [1, 8] or null arrays", ndim);
+    ReduceNdArgs p = {};
+    p.n_out = 1;
+    p.n_red_total = 1;
+    for (int d = 0; d < ndim; ++d) {
+        MI355X_REQUIRE(shape[d] >= 0, "reduce_nd: negative extent");
+        if (reduced[d]) {
+            p.red_shape[p.n_red] = shape[d]; p.red_strides[p.n_red++] = x_strides[d]; p.n_red_total *= shape[d];
+        } else {
+            p.keep_shape[p.n_keep] = shape[d]; p.keep_strides[p.n_keep++] = x_strides[d]; p.n_out *= shape[d];
+        }
+    }
+    MI355X_REQUIRE(p.n_red_total >= 1, "reduce_nd: empty reduction");
+    if (p.n_out == 0) return MI355X_OK;
+    MI355X_REQUIRE(X && Y, "reduce_nd: null pointer");
+    const int64_t blocks = ceil_div(p.n_out, (int64_t)(256 / WAVE));
+    MI355X_REQUIRE(blocks < ((int64_t)1 << 31), "reduce_nd: grid too large");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)blocks), block(256);
+    switch (kind) {
+        case MI355X_REDUCE_MEAN: hipLaunchKernelGGL(reduce_nd<MI355X_REDUCE_MEAN>, grid, block, 0, st, X, Y, p); break;
+        case MI355X_REDUCE_SUM: hipLaunchKernelGGL(reduce_nd<MI355X_REDUCE_SUM>, grid, block, 0, st, X, Y, p); break;
+        case MI355X_REDUCE_MAX: hipLaunchKernelGGL(reduce_nd<MI355X_REDUCE_MAX>, grid, block, 0, st, X, Y, p); break;
+        default: hipLaunchKernelGGL(reduce_nd<MI355X_REDUCE_MIN>, grid, block, 0, st, X, Y, p); break;
+    }
+    return check_launch("reduce_nd");
 }

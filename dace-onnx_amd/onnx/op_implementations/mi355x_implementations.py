@@ -694,30 +694,47 @@ def _reduce_split(node, X):
     return prod(X.shape[:axes[0]]), prod(X.shape[axes[0]:axes[-1] + 1]), prod(X.shape[axes[-1] + 1:]), axes
 
 
+def _reduce_axes(node, X):
+    """Sorted, normalised reduced axes (all of them when the attribute is absent), or None when invalid."""
+    rank = len(X.shape)
+    if node.axes is None:
+        return list(range(rank))
+    if any(not -rank <= a < rank for a in node.axes) or len({a % rank for a in node.axes}) != len(node.axes):
+        return None
+    return sorted(a % rank for a in node.axes)
+
+
 def _reduce_impl(op_name, kind, cite):
     @op_implementation(op=op_name, name=IMPLEMENTATION_NAME)
     class Impl(ONNXForward):
-        __doc__ = (f"{op_name} over ``axes`` (attribute form, opset < 13 / 18) when they are adjacent "
-                   f"({cite}).")
+        __doc__ = (f"{op_name} over ``axes`` (attribute form, opset < 13 / 18): adjacent axes as one axis of the "
+                   f"product length, any other set through the general kernel ({cite}).")
 
         @staticmethod
         def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
             X = in_desc_with_name(node, state, sdfg, "data")
             Y = out_desc_with_name(node, state, sdfg, "reduced")
-            if not _is_f32(X, Y) or not _contig(X, Y) or len(X.shape) < 1:
+            if not _is_f32(X, Y) or not _contig(X, Y) or not 1 <= len(X.shape) <= MAX_ELTWISE_DIMS:
                 return False
-            split = _reduce_split(node, X)
-            if split is None or split[1] < 1:
+            axes = _reduce_axes(node, X)
+            if not axes or prod([X.shape[a] for a in axes]) < 1:
                 return False
             keep = node.keepdims is None or bool(node.keepdims)
-            want = [1 if d in split[3] else e for d, e in enumerate(X.shape)] if keep else \
-                [e for d, e in enumerate(X.shape) if d not in split[3]]
-            return [e for e in Y.shape if e != 1] == [e for e in want if e != 1] and Y.total_size == split[0] * split[2]
+            want = [1 if d in axes else e for d, e in enumerate(X.shape)] if keep else \
+                [e for d, e in enumerate(X.shape) if d not in axes]
+            return [e for e in Y.shape if e != 1] == [e for e in want if e != 1] and \
+                Y.total_size == prod([e for d, e in enumerate(X.shape) if d not in axes])
 
         @staticmethod
         def forward(node, state: SDFGState, sdfg: SDFG):
             X = in_desc_with_name(node, state, sdfg, "data")
-            outer, axis_len, inner, _ = _reduce_split(node, X)
+            split = _reduce_split(node, X)
+            if split is None:       # the reduced axes are not adjacent
+                axes = _reduce_axes(node, X)
+                return kernel_call_for_node(node, state, "mi355x_reduce_nd_f32", [
+                    kind, Ptr("data"), Ptr("reduced"), len(X.shape), I64Array(X.shape), I64Array(X.strides),
+                    I64Array([int(d in axes) for d in range(len(X.shape))]), Stream()])
+            outer, axis_len, inner, _ = split
             if kind == _lib.REDUCE_MEAN:
                 return kernel_call_for_node(node, state, "mi355x_reduce_mean_f32",
                                             [Ptr("data"), Ptr("reduced"), outer, axis_len, inner, Stream()])

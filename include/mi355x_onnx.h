@@ -214,6 +214,13 @@ int mi355x_reduce_f32(int kind, const float* X, float* Y,
                       int64_t outer, int64_t axis_len, int64_t inner,
                       void* stream);
 
+/* The same reductions over any set of axes (ReduceSum over axes 0 and 2 of a [2, 4, 10] tensor, as in the
+ * reference's tests/pure_expansions/test_expansions.py:176-230): `reduced[d]` != 0 marks the axes of
+ * X[shape] (element strides x_strides) that are reduced; Y holds the kept axes in order, C-contiguous. One
+ * wave per output element; adjacent axes are served faster by mi355x_reduce_f32. ndim <= 8. */
+int mi355x_reduce_nd_f32(int kind, const float* X, float* Y, int ndim, const int64_t* shape,
+                         const int64_t* x_strides, const int64_t* reduced, void* stream);
+
 /* Elementwise ops, fp32, with numpy broadcasting.
  * Replaces the one-map expansions Add/Sub/Mul/Div
  * (pure_implementations.py:77-94), PurePow (:59-74), PureRelu (:462-474),

@@ -515,6 +515,110 @@ def test_global_average_pool_and_batch_normalization(shape):
     assert np.allclose(Z, expected, rtol=1e-5, atol=1e-5) and rel_err(expected, Z) < 1e-6
 
 
+def _single_node_sdfg(sdfg_name, node, inputs, out_conn, out_shape, out_dtype=None):
+    """The hand-built one-node SDFG of the reference's expansion tests: arrays, one state, the node, its edges."""
+    sdfg = dace.SDFG(sdfg_name)
+    state = sdfg.add_state()
+    state.add_node(node)
+    for conn, (name, value) in inputs.items():
+        sdfg.add_array(name, list(value.shape), dace.typeclass_of(value.dtype))
+        state.add_edge(state.add_access(name), None, node, conn, sdfg.make_array_memlet(name))
+    sdfg.add_array("__return", list(out_shape), out_dtype or dace.float32)
+    state.add_edge(node, out_conn, state.add_access("__return"), None, sdfg.make_array_memlet("__return"))
+    sdfg.expand_library_nodes()
+    assert_expanded_to_kernels(sdfg)
+    return sdfg
+
+
+@pytest.mark.parametrize("reduce_type, keepdims, axes", [("Sum", True, [0]), ("Sum", False, [-1]), ("Sum", True, [0, -1]),
+                                                         ("Max", False, [0, -1]), ("Max", True, [0]), ("Max", True, [-1]),
+                                                         ("Mean", True, [-1]), ("Mean", True, [0, -1]), ("Mean", False, [0]),
+                                                         ("Min", False, [0, -1]), ("Min", True, [1])])
+def test_reduce(keepdims, reduce_type, axes, sdfg_name):
+    # tests/pure_expansions/test_expansions.py:176-230 (its grid, including the non-adjacent axes [0, -1]), plus Min
+    X = np.random.default_rng(32).normal(scale=10, size=(2, 4, 10)).astype(np.float32)
+    numpy_result = getattr(np, reduce_type.lower())(X.copy(), axis=tuple(axes), keepdims=keepdims)
+    op_node = getattr(donnx, "ONNXReduce" + reduce_type)("reduce")
+    op_node.axes = axes
+    op_node.keepdims = 1 if keepdims else 0
+    sdfg = _single_node_sdfg(sdfg_name, op_node, {"data": ("X", X)}, "reduced", numpy_result.shape)
+    result = sdfg(X=X)
+    assert np.allclose(numpy_result, result, rtol=1e-5, atol=1e-5)
+
+
+def test_reduce_scalar(sdfg_name):
+    # tests/pure_expansions/test_expansions.py:233-270: no axes attribute, keepdims 0 -> every axis, one value
+    X = np.random.default_rng(33).normal(scale=10, size=(2, 4, 10)).astype(np.float32)
+    op_node = donnx.ONNXReduceMean("mean")
+    op_node.keepdims = 0
+    sdfg = _single_node_sdfg(sdfg_name, op_node, {"data": ("X", X)}, "reduced", ())
+    assert np.allclose(np.mean(X), sdfg(X=X))
+
+
+@pytest.mark.parametrize("shape, axes", [((6, 5, 7, 3), [0, 2]), ((6, 5, 7, 3), [1, 3]), ((3, 130, 4, 70), [1, 3]),
+                                         ((2, 3, 4, 5, 6), [0, 2, 4])])
+@pytest.mark.parametrize("op", ["ReduceSum", "ReduceMax", "ReduceMin", "ReduceMean"])
+def test_reduce_non_adjacent_axes(op, shape, axes):
+    X = np.random.default_rng(34).normal(1.0, 2.0, size=shape).astype(np.float32)
+    oracle = {"ReduceSum": O.reduce_sum, "ReduceMax": O.reduce_max, "ReduceMin": O.reduce_min, "ReduceMean": O.reduce_mean}[op]
+    for keepdims in (0, 1):
+        expected = oracle(X.astype(np.float64), axes, keepdims)
+        Y = np.zeros(expected.shape, np.float32)
+        getattr(donnx, "ONNX" + op)(data=X, reduced=Y, axes=axes, keepdims=keepdims)
+        if op in ("ReduceMax", "ReduceMin"):
+            assert np.array_equal(expected.astype(np.float32), Y)
+        else:
+            assert np.allclose(Y, expected, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("src, dst", [(np.int32, np.float32), (np.float32, np.int32), (np.float32, np.int64)])
+def test_cast_reference_cases(src, dst, sdfg_name):
+    # tests/pure_expansions/test_expansions.py:78-174: int -> float, float -> int, float -> long on a [2, 4, 10] array
+    X = np.random.default_rng(35).normal(scale=10, size=(2, 4, 10)).astype(src)
+    op_node = donnx.ONNXCast("Cast", to=proto.np_dtype_to_tensor_dtype(np.dtype(dst)))   # `to` is a required attribute
+    sdfg = _single_node_sdfg(sdfg_name, op_node, {"input": ("X", X)}, "output", X.shape, dace.typeclass_of(np.dtype(dst)))
+    result = sdfg(X=X)
+    assert result.dtype == np.dtype(dst) and np.array_equal(X.astype(dst), result)
+
+
+def test_cast_scalar():
+    # tests/pure_expansions/test_expansions.py:61-75: a float64 scalar to float32
+    out = np.zeros((), np.float32)
+    donnx.ONNXCast(input=np.array(2.0, np.float64), output=out, to=proto.np_dtype_to_tensor_dtype(np.dtype(np.float32)))
+    assert out == 2
+
+
+@pytest.mark.parametrize("shape", [(2, 3), (1, ), ()])
+def test_sum_arrays(shape):
+    # tests/pure_expansions/test_expansions.py:500-530: three inputs of one shape, also [1] and scalars
+    rng = np.random.default_rng(36)
+    inputs = [np.asarray(rng.normal(size=shape), dtype=np.float32) for _ in range(3)]
+    result = np.zeros(shape, np.float32)
+    donnx.ONNXSum(data_0__0=inputs[0], data_0__1=inputs[1], data_0__2=inputs[2], sum=result)
+    assert np.allclose(result, (inputs[0] + inputs[1]) + inputs[2])
+
+
+def test_reshape_then_add():
+    # tests/pure_expansions/test_expansions.py:477-497: Reshape whose target is a run-time input; the result's shape
+    # is the declared one
+    inp, bias = np.arange(9).astype(np.float32), np.arange(3).astype(np.float32)
+    reshaped, out = np.zeros((3, 3), np.float32), np.zeros((3, 3), np.float32)
+    donnx.ONNXReshape(data=inp, shape=np.array([3, 3]).astype(np.int64), reshaped=reshaped)
+    donnx.ONNXAdd(A=reshaped, B=bias, C=out)
+    assert np.allclose(out, inp.reshape(3, 3) + bias)
+
+
+def test_reciprocal_and_logsoftmax_reference_cases(sdfg_name):
+    # tests/pure_expansions/test_expansions.py:384-453
+    X = np.random.default_rng(37).normal(scale=10, size=(2, 4, 10)).astype(np.float32)
+    for axis in (0, 1, 2, -1):
+        Y = np.zeros_like(X)
+        donnx.ONNXLogSoftmax(input=X, output=Y, axis=axis)
+        assert np.linalg.norm(torch.nn.functional.log_softmax(torch.from_numpy(X), dim=axis).numpy() - Y) < 1e-5
+    sdfg = _single_node_sdfg(sdfg_name, donnx.ONNXReciprocal("reciprocal"), {"X": ("X", X)}, "Y", X.shape)
+    assert np.allclose(1 / X, sdfg(X=X))
+
+
 def test_pow():
     rng = np.random.default_rng(16)
     X = rng.normal(size=(8, 16, 64)).astype(np.float32)

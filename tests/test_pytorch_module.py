@@ -143,6 +143,28 @@ def test_conv_batchnorm_pool_network_results(exporter):
     assert rel_err(ref.numpy(), plain(x.cuda()).cpu().numpy()) < FP32_REL_TOL
 
 
+class _LogSqrt(nn.Module):
+    """The example of the reference's DaceModule docstring (daceml/pytorch/module.py:43-55)."""
+    def forward(self, x):
+        x = torch.log(x)
+        x = torch.sqrt(x)
+        return x
+
+
+def test_docstring_example_is_one_launch():
+    dm = DaceModule(_LogSqrt(), dummy_inputs=(torch.ones(2), ))
+    assert [n.op_type for n in dm.onnx_model.graph.node] == ["Log", "Sqrt"]
+    assert _functions(dm) == ["mi355x_eltwise_program_f32"]
+
+
+@pytest.mark.gpu
+def test_docstring_example_result():
+    dace_module = DaceModule(_LogSqrt())
+    assert dace_module(torch.ones(2).cuda()).tolist() == [0.0, 0.0]
+    x = torch.rand(7, 5) + 1.0
+    assert torch.allclose(dace_module.model(x), DaceModule(_LogSqrt())(x.cuda()).cpu(), rtol=1e-6, atol=1e-7)
+
+
 class _ResidualBlock(nn.Module):
     """A ResNet basic block with a projection shortcut (not a Sequential: only the exporter can write it)."""
     def __init__(self, c):
