@@ -143,6 +143,78 @@ def test_conv_batchnorm_pool_network_results(exporter):
     assert rel_err(ref.numpy(), plain(x.cuda()).cpu().numpy()) < FP32_REL_TOL
 
 
+class _LeNet(nn.Module):
+    """The network of the reference's tests/pytorch/test_lenet.py:14-34."""
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(1, 6, (3, 3))
+        self.conv2 = nn.Conv2d(6, 16, (3, 3))
+        self.fc1 = nn.Linear(16 * 6 * 6, 120)
+        self.fc2 = nn.Linear(120, 84)
+        self.fc3 = nn.Linear(84, 10)
+
+    def forward(self, x):
+        F = torch.nn.functional
+        x = F.max_pool2d(F.relu(self.conv1(x)), 2)
+        x = F.max_pool2d(F.relu(self.conv2(x)), 2)
+        x = x.view(-1, 16 * 6 * 6)
+        x = F.relu(self.fc1(x))
+        x = F.relu(self.fc2(x))
+        x = self.fc3(x)
+        return F.log_softmax(x, dim=1)
+
+
+def test_lenet_launch_list():
+    dm = DaceModule(_LeNet(), dummy_inputs=(torch.rand(8, 1, 32, 32), ))
+    assert [n.op_type for n in dm.onnx_model.graph.node] == ["Conv", "Relu", "MaxPool", "Conv", "Relu", "MaxPool", "Constant",
+                                                             "Reshape", "Gemm", "Relu", "Gemm", "Relu", "Gemm", "LogSoftmax"]
+    # every Relu rides in the epilogue of the Conv / Gemm before it, the view is free
+    assert _functions(dm) == ["mi355x_conv2d_f32", "mi355x_maxpool2d_f32", "mi355x_conv2d_f32", "mi355x_maxpool2d_f32",
+                              "mi355x_gemm_f32", "mi355x_gemm_f32", "mi355x_gemm_f32", "mi355x_log_softmax_f32"]
+
+
+@pytest.mark.gpu
+def test_lenet(sdfg_name):
+    # tests/pytorch/test_lenet.py:37-57
+    torch.manual_seed(7)
+    input = torch.rand(8, 1, 32, 32, dtype=torch.float32)
+    net = _LeNet()
+    dace_net = _LeNet()
+    dace_net.load_state_dict(net.state_dict())
+    dace_net = DaceModule(dace_net, sdfg_name=sdfg_name)
+    torch_output = net(torch.clone(input))
+    dace_output = dace_net(torch.clone(input).cuda())
+    torch_tensors_close("output", torch_output, dace_output.cpu())
+
+
+class _ReshapeModel(nn.Module):
+    def __init__(self, new_shape):
+        super().__init__()
+        self.new_shape = new_shape
+
+    def forward(self, x):
+        return x.reshape(self.new_shape)
+
+
+@pytest.mark.gpu
+def test_reshape_module_global_avg_pool_and_batchnorm(sdfg_name):
+    # tests/pytorch/test_reshape.py:19-34
+    x = torch.rand([25])
+    dace_model = DaceModule(_ReshapeModel([5, 5]), auto_optimize=False, dummy_inputs=(x, ), sdfg_name=sdfg_name)
+    torch_tensors_close("output", x.reshape(5, 5), dace_model(x.cuda()).cpu())
+    # tests/pytorch/test_img_op_implementations.py:36-49
+    inputs = torch.rand(1, 64, 60, 60)
+    torch_tensors_close("output", nn.AdaptiveAvgPool2d(1)(inputs), DaceModule(nn.AdaptiveAvgPool2d(1))(inputs.cuda()).cpu())
+    # ... :12-33 in inference form (the reference's test runs BatchNorm2d in training mode, which is not provided here)
+    bn = nn.BatchNorm2d(64).eval()
+    with torch.no_grad():
+        bn.running_mean.normal_()
+        bn.running_var.uniform_(0.5, 2.0)
+    torch_tensors_close("output", bn(inputs), DaceModule(bn)(inputs.cuda()).cpu())
+    with pytest.raises(NotImplementedError, match="inference only"):
+        DaceModule(nn.BatchNorm2d(64), training=True)
+
+
 class _LogSqrt(nn.Module):
     """The example of the reference's DaceModule docstring (daceml/pytorch/module.py:43-55)."""
     def forward(self, x):
