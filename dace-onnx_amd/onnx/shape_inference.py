@@ -206,7 +206,10 @@ def infer_shapes(model: ModelProto) -> ModelProto:
             if out_name not in known_vi:
                 g.value_info.append(ValueInfoProto(out_name, ty, list(shape)))
                 known_vi.add(out_name)
-    for v in g.output:
-        if v.shape is None and v.name in shapes:
+    # an output (or intermediate) declared without a shape, or with symbolic dimensions -- exporters write those
+    # when their own inference gives up on computed pads / targets -- takes the inferred static shape
+    for v in list(g.output) + list(g.value_info):
+        static = v.shape is not None and all(isinstance(d, int) for d in v.shape)
+        if not static and v.name in shapes:
             v.shape, v.elem_type = list(shapes[v.name]), types[v.name]
     return model

@@ -480,3 +480,12 @@ def test_conv_residual_epilogue(shape, wshape, pads, strides, epi):
     args[3] = None
     assert lib.mi355x_conv2d_res_f32(*args) == 1 and b"without residual" in lib.mi355x_last_error()
     assert lib.mi355x_conv2d_f32(*(args[:3] + args[4:-2] + [_lib.EPI_RESIDUAL, None])) == 1
+
+
+def test_tasklet_fusion_programs_values():
+    # tests/transformation/test_tasklet_fusion.py:9-60 of the reference: same inputs (ones, twos), same expectations
+    from test_fusion import _tasklet_fusion_graphs
+    A, B = np.ones((5, 5), np.float32), np.ones((5, 5), np.float32) * 2
+    for name, (m, inputs, fn) in _tasklet_fusion_graphs().items():
+        result = donnx.ONNXModel("tf_values_" + name, m)(*([A, B][:len(inputs)]))
+        assert np.allclose(result, fn(A, B)), name

@@ -350,3 +350,30 @@ def test_batchnorm_folds_into_the_convolution():
         assert "mi355x_batchnorm_f32" in [f for f, _ in calls]
     unfused = _launches(donnx.ONNXModel("conv_bn_plain", _conv_bn_model()[0], fuse=False))
     assert [f for f, _ in unfused] == ["mi355x_conv2d_f32", "mi355x_batchnorm_f32", "mi355x_eltwise_f32"]
+
+
+def _tasklet_fusion_graphs():
+    """The three programs of the reference's tests/transformation/test_tasklet_fusion.py, as ONNX graphs:
+    (A + 1) * 2, (A + 1) + (A * 3), (A + 1) + (B * 3)."""
+    mk, T = H.make_node, proto.TensorProto
+    consts = [proto.numpy_helper.from_array(np.array(v, np.float32), k) for k, v in (("one", 1.0), ("two", 2.0), ("three", 3.0))]
+    graphs = {
+        "basic": ([mk("Add", ["A", "one"], ["b"]), mk("Mul", ["b", "two"], ["y"])], ["A"], lambda A, B: (A + 1) * 2),
+        "same_name": ([mk("Add", ["A", "one"], ["b"]), mk("Mul", ["A", "three"], ["c"]), mk("Add", ["b", "c"], ["y"])], ["A"],
+                      lambda A, B: A + 1 + A * 3),
+        "same_name_diff_memlet": ([mk("Add", ["A", "one"], ["d"]), mk("Mul", ["B", "three"], ["c"]), mk("Add", ["d", "c"], ["y"])],
+                                  ["A", "B"], lambda A, B: A + 1 + B * 3),
+    }
+    out = {}
+    for name, (nodes, inputs, fn) in graphs.items():
+        g = H.make_graph(nodes, name, [H.make_tensor_value_info(i, T.FLOAT, [5, 5]) for i in inputs],
+                         [H.make_tensor_value_info("y", T.FLOAT, [5, 5])], initializer=consts)
+        out[name] = (H.make_model(g, opset_imports=[H.make_opsetid("", 12)]), inputs, fn)
+    return out
+
+
+def test_tasklet_fusion_programs_become_one_launch():
+    for name, (m, inputs, _) in _tasklet_fusion_graphs().items():
+        calls = _launches(donnx.ONNXModel("tf_" + name, m))
+        assert [f for f, _ in calls] == ["mi355x_eltwise_program_f32"], name
+        assert calls[0][1][1] == len(inputs) and calls[0][1][8] == len(m.graph.node)     # tensors read, instructions

@@ -215,6 +215,64 @@ def test_reshape_module_global_avg_pool_and_batchnorm(sdfg_name):
         DaceModule(nn.BatchNorm2d(64), training=True)
 
 
+class _PadConv(nn.Module):
+    """tests/transformation/test_pad_conv_fusion.py:13-20 of the reference."""
+    def __init__(self):
+        super().__init__()
+        self.conv = nn.Conv2d(3, 6, kernel_size=(3, 3))
+
+    def forward(self, x):
+        return self.conv(torch.nn.functional.pad(x, [2, 2]))
+
+
+class _ConvPoolViewRelu(nn.Module):
+    """tests/transformation/test_reshape_elimination.py:12-20 of the reference."""
+    def __init__(self):
+        super().__init__()
+        self.conv = nn.Conv2d(6, 16, 5)
+
+    def forward(self, x):
+        F = torch.nn.functional
+        x = F.max_pool2d(F.relu(self.conv(x)), 2)
+        return F.relu(x.view(-1, 256))
+
+
+class _AddTwo(nn.Module):
+    """tests/transformation/test_input_to_constant.py:13-19 of the reference (an unused parameter, a scalar constant)."""
+    def __init__(self):
+        super().__init__()
+        self.fc1 = nn.Linear(5, 3)
+
+    def forward(self, x):
+        return x + 2
+
+
+_TRANSFORMATION_TEST_MODULES = [(_PadConv, (4, 3, 24, 24), ["mi355x_conv2d_f32"]),
+                                (_ConvPoolViewRelu, (100, 6, 12, 12), ["mi355x_conv2d_f32", "mi355x_maxpool2d_f32", "mi355x_eltwise_f32"]),
+                                (_AddTwo, (10, 5), ["mi355x_eltwise_f32"])]
+
+
+@pytest.mark.parametrize("cls, shape, launches", _TRANSFORMATION_TEST_MODULES)
+def test_transformation_test_modules_launch_lists(cls, shape, launches):
+    # the exporter's pad arithmetic (a dozen shape nodes) folds to a constant, the Pad into the convolution's pads --
+    # the output's symbolic declared shape is replaced by the inferred one; views cost nothing
+    dm = DaceModule(cls(), dummy_inputs=(torch.rand(*shape), ))
+    assert _functions(dm) == launches
+    if cls is _PadConv:
+        call = [n for n, _ in dm.dace_model.sdfg.all_nodes_recursive() if isinstance(n, dace.KernelCall)][0]
+        assert [0, 2, 0, 2] in [getattr(a, "values", None) for a in call.args]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cls, shape, launches", _TRANSFORMATION_TEST_MODULES)
+def test_transformation_test_modules_results(cls, shape, launches):
+    torch.manual_seed(8)
+    torch_module = cls()
+    dace_module = DaceModule(copy.deepcopy(torch_module))
+    input = torch.rand(*shape)
+    torch_tensors_close("output", torch_module(input), dace_module(input.cuda()).cpu())
+
+
 class _LogSqrt(nn.Module):
     """The example of the reference's DaceModule docstring (daceml/pytorch/module.py:43-55)."""
     def forward(self, x):
