@@ -532,7 +532,7 @@ class MI355XBatchNormalization(ONNXForward):
         Y = out_desc_with_name(node, state, sdfg, "Y")
         if not _is_f32(X, Y) or not _contig(X, Y) or len(X.shape) < 2 or tuple(X.shape) != tuple(Y.shape):
             return False
-        for conn in ("scale", "B", "mean", "var"):
+        for conn in ("scale", "B", "in_mean", "in_var"):
             if not _has_input(node, state, conn):
                 return False
             d = in_desc_with_name(node, state, sdfg, conn)
@@ -545,7 +545,7 @@ class MI355XBatchNormalization(ONNXForward):
         X = in_desc_with_name(node, state, sdfg, "X")
         eps = 1e-5 if node.epsilon is None else float(node.epsilon)
         return kernel_call_for_node(node, state, "mi355x_batchnorm_f32", [
-            Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("mean"), Ptr("var"), Ptr("Y"), X.shape[0], X.shape[1],
+            Ptr("X"), Ptr("scale"), Ptr("B"), Ptr("in_mean"), Ptr("in_var"), Ptr("Y"), X.shape[0], X.shape[1],
             prod(X.shape[2:]), eps, Stream()])
 
 

@@ -182,12 +182,13 @@ SCHEMAS: typing.List[ONNXSchema] = [
                "Max pooling over sliding windows."),
     _unary("GlobalAveragePool", 1, "X", "Y", doc="Mean over the spatial axes."),
     ONNXSchema("BatchNormalization", 9,
-               [ONNXParameter("X", "T"), ONNXParameter("scale", "T"), ONNXParameter("B", "T"), ONNXParameter("mean", "T"),
-                ONNXParameter("var", "T")],
+               [ONNXParameter("X", "T"), ONNXParameter("scale", "T"), ONNXParameter("B", "T"), ONNXParameter("in_mean", "T"),
+                ONNXParameter("in_var", "T")],
                [ONNXParameter("Y", "T"), ONNXParameter("out_mean", "T", _O), ONNXParameter("out_var", "T", _O),
                 ONNXParameter("saved_mean", "T", _O), ONNXParameter("saved_var", "T", _O)],
                [ONNXAttribute("epsilon", _A.Float, 1e-5), ONNXAttribute("momentum", _A.Float, 0.9)],
-               [ONNXTypeConstraint("T", _FLOATS)], "Batch normalization."),
+               [ONNXTypeConstraint("T", _FLOATS)], "Batch normalization. ONNX names the statistics `mean` / `var` on both sides; as in the reference "
+               "(onnx_op.py:499-508) the inputs are `in_mean` / `in_var` and the outputs `out_mean` / `out_var`."),
     ONNXSchema("Sum", 8, [ONNXParameter("data_0", "T", ONNXParameterType.Variadic)], [ONNXParameter("sum", "T")], (),
                [ONNXTypeConstraint("T", _FLOATS)], "Elementwise sum of the inputs."),
 ]

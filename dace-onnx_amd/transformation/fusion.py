@@ -226,7 +226,7 @@ def _fold_batchnorm_into_conv(sdfg: SDFG, state: SDFGState) -> int:
         if len(state.out_edges(bn)) != 1 or _out_edge(state, bn, "Y") is None:
             continue        # training outputs present
         w = constant(conv, "W")
-        params = [constant(bn, c) for c in ("scale", "B", "mean", "var")]
+        params = [constant(bn, c) for c in ("scale", "B", "in_mean", "in_var")]
         has_bias = _in_edge(state, conv, "B") is not None
         bias = constant(conv, "B") if has_bias else None
         if w is None or any(p is None for p in params) or (has_bias and bias is None):

@@ -510,7 +510,7 @@ def test_global_average_pool_and_batch_normalization(shape):
     scale, b, mean = (rng.normal(size=C).astype(np.float32) for _ in range(3))
     var = rng.uniform(0.5, 2.0, size=C).astype(np.float32)
     Z = np.zeros_like(X)
-    donnx.ONNXBatchNormalization(X=X, scale=scale, B=b, mean=mean, var=var, Y=Z, epsilon=1e-3)
+    donnx.ONNXBatchNormalization(X=X, scale=scale, B=b, in_mean=mean, in_var=var, Y=Z, epsilon=1e-3)
     expected = O.batch_normalization(X, scale, b, mean, var, 1e-3)
     assert np.allclose(Z, expected, rtol=1e-5, atol=1e-5) and rel_err(expected, Z) < 1e-6
 
@@ -617,6 +617,19 @@ def test_reciprocal_and_logsoftmax_reference_cases(sdfg_name):
         assert np.linalg.norm(torch.nn.functional.log_softmax(torch.from_numpy(X), dim=axis).numpy() - Y) < 1e-5
     sdfg = _single_node_sdfg(sdfg_name, donnx.ONNXReciprocal("reciprocal"), {"X": ("X", X)}, "Y", X.shape)
     assert np.allclose(1 / X, sdfg(X=X))
+
+
+def test_bn_standalone():
+    # tests/test_shared_input_output.py:17-41 of the reference: `mean` / `var` name an input and an output of the ONNX
+    # operator, so the connectors are in_mean / in_var (and out_mean / out_var)
+    X, scale, B, mean = torch.randn(8, 3, 32, 32), torch.randn(3), torch.randn(3), torch.randn(3)
+    var = torch.rand(3) + 0.5
+    Y = np.zeros((8, 3, 32, 32), np.float32)
+    donnx.ONNXBatchNormalization(X=X.numpy(), scale=scale.numpy(), B=B.numpy(), in_mean=mean.numpy(), in_var=var.numpy(), Y=Y)
+    pt_result = torch.nn.functional.batch_norm(X, mean, var, scale, B)
+    assert np.allclose(pt_result.numpy(), Y, rtol=1e-5, atol=1e-4)
+    with pytest.raises(TypeError, match="Unknown arguments"):
+        donnx.ONNXBatchNormalization(X=X.numpy(), scale=scale.numpy(), B=B.numpy(), mean=mean.numpy(), var=var.numpy(), Y=Y)
 
 
 def test_pow():

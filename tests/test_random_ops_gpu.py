@@ -93,7 +93,7 @@ def test_random_operator_cases(seed):
     scale, b, mean = (rng.normal(size=C).astype(np.float32) for _ in range(3))
     var = rng.uniform(0.1, 3.0, size=C).astype(np.float32)
     Z = np.zeros_like(X)
-    donnx.ONNXBatchNormalization(X=X, scale=scale, B=b, mean=mean, var=var, Y=Z, epsilon=1e-5)
+    donnx.ONNXBatchNormalization(X=X, scale=scale, B=b, in_mean=mean, in_var=var, Y=Z, epsilon=1e-5)
     check(f"BatchNormalization {X.shape}", np.allclose(Z, O.batch_normalization(X, scale, b, mean, var, 1e-5), rtol=2e-5, atol=2e-5))
     G = np.zeros(X.shape[:2] + (1, 1), np.float32)
     donnx.ONNXGlobalAveragePool(X=X, Y=G)
