@@ -136,7 +136,7 @@ def register(ops: typing.Optional[typing.Iterable[str]] = None) -> typing.List[s
     for op in (ops or ["MatMul", "Gemm", "Conv", "MatMulInteger", "Softmax", "Add", "Sub", "Mul", "Div", "Pow", "Relu", "Erf",
                        "Sqrt", "Log", "Tanh", "Sigmoid", "Softplus", "Reciprocal", "Exp", "Neg", "Abs", "ReduceMean", "ReduceSum",
                        "ReduceMax", "ReduceMin", "LogSoftmax", "Sum", "Cast", "Slice", "Einsum", "MaxPool", "GlobalAveragePool",
-                       "BatchNormalization", "Transpose"]):
+                       "BatchNormalization", "Squeeze", "Unsqueeze", "Transpose"]):
         dace_node = getattr(donnx, "ONNX" + op, None)
         if dace_node is None:
             continue

@@ -995,6 +995,9 @@ def _alias_impl(op_name, in_conn, out_conn):
 MI355XReshape = _alias_impl("Reshape", "data", "reshaped")
 MI355XFlatten = _alias_impl("Flatten", "input", "output")
 MI355XIdentity = _alias_impl("Identity", "input", "output")
+# Squeeze / Unsqueeze have no pure expansion in the reference (ONNX Runtime copies the data there)
+MI355XSqueeze = _alias_impl("Squeeze", "data", "squeezed")
+MI355XUnsqueeze = _alias_impl("Unsqueeze", "data", "expanded")
 
 
 @op_implementation(op="Pad", name=IMPLEMENTATION_NAME)

@@ -136,6 +136,8 @@ SCHEMAS: typing.List[ONNXSchema] = [
     _unary("Transpose", 1, "data", "transposed", types=_ANY, attributes=[ONNXAttribute("perm", _A.Ints)]),
     _unary("Flatten", 11, "input", "output", types=_ANY, attributes=[ONNXAttribute("axis", _A.Int, 1)]),
     _unary("Identity", 1, "input", "output", types=_ANY),
+    _unary("Squeeze", 11, "data", "squeezed", types=_ANY, attributes=[ONNXAttribute("axes", _A.Ints)]),
+    _unary("Unsqueeze", 11, "data", "expanded", types=_ANY, attributes=[ONNXAttribute("axes", _A.Ints, required=True)]),
     # Pad only ever runs folded into the Conv that reads it (transformation/fusion.py, the reference's PadConvFusion)
     ONNXSchema("Pad", 11,
                [ONNXParameter("data", "T"), ONNXParameter("pads", "tensor(int64)"), ONNXParameter("constant_value", "T", _O)],

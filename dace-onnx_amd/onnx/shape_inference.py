@@ -125,6 +125,19 @@ def _infer_node(node, shapes, types, constants):
     if op == "Flatten":
         axis = a.get("axis", 1) % (len(ins[0]) + 1) if a.get("axis", 1) < 0 else a.get("axis", 1)
         return [((int(np.prod(ins[0][:axis])) if axis else 1, int(np.prod(ins[0][axis:]))), tys[0])]
+    if op == "Squeeze":
+        rank = len(ins[0])
+        axes = [ax % rank for ax in a["axes"]] if a.get("axes") is not None else [i for i, d in enumerate(ins[0]) if d == 1]
+        if any(ins[0][ax] != 1 for ax in axes):
+            raise ShapeInferenceError(f"Squeeze '{node.name}': axes {axes} of {ins[0]} are not all of extent 1")
+        return [(tuple(d for i, d in enumerate(ins[0]) if i not in axes), tys[0])]
+    if op == "Unsqueeze":
+        rank = len(ins[0]) + len(a["axes"])
+        axes = sorted(ax % rank for ax in a["axes"])
+        out = list(ins[0])
+        for ax in axes:
+            out.insert(ax, 1)
+        return [(tuple(out), tys[0])]
     if op == "Cast":
         return [(ins[0], int(a["to"]))]
     if op == "Slice":

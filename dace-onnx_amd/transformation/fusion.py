@@ -408,7 +408,7 @@ def _input_view(sdfg, state, access: AccessNode):
         if _is_op(n, "Transpose"):
             chain.append(("T", n))
             cur = _in_edge(state, n, "data").src
-        elif _is_op(n, "Reshape"):
+        elif _is_op(n, "Reshape", "Squeeze", "Unsqueeze"):     # all three: the same elements under another shape
             chain.append(("R", n))
             cur = _in_edge(state, n, "data").src
         else:
@@ -426,7 +426,7 @@ def _input_view(sdfg, state, access: AccessNode):
             perm = list(n.perm) if n.perm is not None else list(reversed(range(len(shape))))
             shape, strides = [shape[p] for p in perm], [strides[p] for p in perm]
         else:
-            new_shape = list(sdfg.arrays[_out_edge(state, n, "reshaped").dst.data].shape)
+            new_shape = list(sdfg.arrays[_out_edge(state, n, n.schema.outputs[0].name).dst.data].shape)
             new_strides = _reshape_strides(shape, strides, new_shape)
             if new_strides is None:
                 return None
@@ -1215,7 +1215,7 @@ def _remove_dead_nodes(sdfg: SDFG, state: SDFGState) -> int:
                 if desc is not None and desc.transient and not state.out_edges(n) and state.in_edges(n):
                     prod = state.in_edges(n)[0].src
                     # only pure data-movement nodes are dropped; anything else would be a graph bug
-                    if _is_op(prod, "Transpose", "Reshape", "Identity", "Flatten") and len(state.out_edges(prod)) == 1:
+                    if _is_op(prod, "Transpose", "Reshape", "Identity", "Flatten", "Squeeze", "Unsqueeze") and len(state.out_edges(prod)) == 1:
                         state.remove_node(prod)
                         state.remove_node(n)
                         del sdfg.arrays[n.data]

@@ -96,5 +96,6 @@ def test_model_without_constant_subgraphs_is_returned_as_is_and_switch_is_honour
     assert fold_constants(plain) is plain
     folded = donnx.ONNXModel("folded", model)
     assert "cu" in folded.weights and len(model.graph.node) == 2      # caller's model untouched
-    with pytest.raises(ValueError, match="Unsupported ONNX operator: 'Unsqueeze'"):
-        donnx.ONNXModel("not_folded", model, fold_constants=False)
+    # with the switch off the Unsqueeze stays a node of the graph (a view at run time)
+    kept = donnx.ONNXModel("not_folded", model, fold_constants=False)
+    assert "cu" not in kept.weights and any(type(n).__name__ == "ONNXUnsqueeze" for n, _ in kept.sdfg.all_nodes_recursive())

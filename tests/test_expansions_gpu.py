@@ -619,6 +619,32 @@ def test_reciprocal_and_logsoftmax_reference_cases(sdfg_name):
     assert np.allclose(1 / X, sdfg(X=X))
 
 
+@pytest.mark.parametrize("shape, axes", [((1, ), None), ((1, ), [0]), ((3, 1, 5, 1), [1, 3]), ((3, 1, 5, 1), [-1]), ((3, 1, 5, 1), None)])
+def test_squeeze_then_unsqueeze(shape, axes, sdfg_name):
+    # tests/test_input_outputs.py:43-95 of the reference: Squeeze an array (there: of one element, to a scalar) and
+    # Unsqueeze it back, as views of the same storage
+    X = np.random.default_rng(38).random(shape).astype(np.float32)
+    squeezed_shape = np.squeeze(X, axis=tuple(axes) if axes is not None else None).shape
+    back_axes = sorted(a % len(shape) for a in axes) if axes is not None else [i for i, d in enumerate(shape) if d == 1]
+    sdfg = dace.SDFG(sdfg_name)
+    sdfg.add_array("X_arr", list(shape), dace.float32)
+    sdfg.add_transient("squeezed", list(squeezed_shape), dace.float32)
+    sdfg.add_array("__return", list(shape), dace.float32)
+    state = sdfg.add_state()
+    sq = donnx.ONNXSqueeze("Squeeze", **({"axes": axes} if axes is not None else {}))
+    unsq = donnx.ONNXUnsqueeze("Unsqueeze", axes=back_axes)
+    mid = state.add_access("squeezed")
+    state.add_node(sq)
+    state.add_node(unsq)
+    state.add_edge(state.add_access("X_arr"), None, sq, "data", sdfg.make_array_memlet("X_arr"))
+    state.add_edge(sq, "squeezed", mid, None, sdfg.make_array_memlet("squeezed"))
+    state.add_edge(mid, None, unsq, "data", sdfg.make_array_memlet("squeezed"))
+    state.add_edge(unsq, "expanded", state.add_access("__return"), None, sdfg.make_array_memlet("__return"))
+    sdfg.expand_library_nodes()
+    assert_expanded_to_kernels(sdfg)
+    assert np.array_equal(sdfg(X_arr=X), X)
+
+
 def test_bn_standalone():
     # tests/test_shared_input_output.py:17-41 of the reference: `mean` / `var` name an input and an output of the ONNX
     # operator, so the connectors are in_mean / in_var (and out_mean / out_var)
