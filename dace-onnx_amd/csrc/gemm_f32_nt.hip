@@ -48,11 +48,13 @@ constexpr int NT_BK = 32, NT_THREADS = 512, NT_RING = 6, NT_STAGES = 3;
 // TN: 16-column MFMA tiles per wave (BN = 16 TN). WAVES_M wave rows of 16 rows each
 // (BM = 16 WAVES_M) times KSPLIT k-split groups make the 8 waves of a workgroup:
 // (4, 2) for problems with few tiles, (8, 1) for 128-row tiles without a reduction.
-// BK: k extent of a tile (32, or 64 where registers allow: half as many barriers per FLOP).
-template <int TN, int WAVES_M, int KSPLIT, int BK = NT_BK>
+// BK: k extent of a tile (32, or 64 where registers allow: half as many barriers per FLOP); RING: k-tiles in
+// flight per lane (six of 32 k or three of 64 k: the same bytes).
+template <int TN, int WAVES_M, int KSPLIT, int BK = NT_BK, int RING = NT_RING>
 __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     static_assert(WAVES_M * KSPLIT * WAVE == NT_THREADS, "8 waves per workgroup");
-    constexpr int BM = 16 * WAVES_M, BN = 16 * TN, RING = NT_RING, NT_PITCH = BK + LDS_PAD;
+    static_assert(RING % NT_STAGES == 0, "a tile's LDS buffer is its ring slot modulo the number of buffers");
+    constexpr int BM = 16 * WAVES_M, BN = 16 * TN, NT_PITCH = BK + LDS_PAD;
     constexpr int NC = (BK / 16) / KSPLIT;  // 16-k chunks of a tile this wave multiplies
     constexpr int B_VECS = BN * (BK / 4);                       // 16-byte vectors of one B tile
     constexpr int B_PER_T = (B_VECS + NT_THREADS - 1) / NT_THREADS;
@@ -281,12 +283,15 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     p.group_m = choose_group_m(p.tiles_m, per_xcd < cus / NUM_XCD ? per_xcd : cus / NUM_XCD, cands[best].bm, cands[best].bn);
     if (const char* g = getenv("MI355X_GEMM_GROUP_M")) p.group_m = atoi(g) > 0 ? atoi(g) : 1;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
-    // 64-k tiles for the smallest variant when K is long: half the barriers per FLOP (42.9 us against 44.8 us
-    // at 1024 x 768 x 3072), but the six-tile prologue then covers 384 k, which costs more than it saves at K = 768
+    // The smallest variant walks K in 64-k tiles with a three-deep ring where K allows: half the barriers per FLOP
+    // and the same bytes in flight as six 32-k tiles (1024 x 768 x 768: 14.0 us against 14.7 us, 1024 x 768 x 3072:
+    // 41.9 us against 44.8 us with 32-k tiles and 43.9 us with six 64-k tiles in flight; the wider
+    // variants lose 1-2 % with 64-k tiles)
     const char* fbk = getenv("MI355X_GEMM_NT_BK");
-    const bool bk64 = p.K % 64 == 0 && (fbk ? atoi(fbk) == 64 : p.K >= 2048);
-    if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64>), grid, block, 0, stream, p);
+    const bool bk64 = p.K % 64 == 0 && (fbk ? atoi(fbk) == 64 : true);
+    if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64, 3>), grid, block, 0, stream, p);
     else if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
+    else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
     else if (best == 2) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((gemm_f32_nt_kernel<9, 4, 2>), grid, block, 0, stream, p);
