@@ -97,22 +97,18 @@ __global__ __launch_bounds__(256) void eltwise_program_kernel(ProgramArgs p) {
         auto fetch = [&](uint32_t enc) __attribute__((always_inline)) -> V {
             const uint32_t idx = enc & 63u;
             V out = L::splat(0.f);
+            // scalar branches, one taken: the empty asm keeps the compiler from turning the cases into a chain of
+            // per-lane selects over every candidate register
+#define MI355X_PICK(arr, n)                                                   \
+            _Pragma("unroll") for (int k = 0; k < (n); ++k)                   \
+                if (idx == (uint32_t)k) { out = arr[k]; asm volatile(""); }
             switch (enc >> 6) {  // uniform
-                case MI355X_PROGRAM_REG:
-#pragma unroll
-                    for (int k = 0; k < NR; ++k) if (idx == (uint32_t)k) out = r[k];
-                    break;
-                case MI355X_PROGRAM_TENSOR:
-#pragma unroll
-                    for (int k = 0; k < NT; ++k) if (idx == (uint32_t)k) out = t[k];
-                    break;
-                case MI355X_PROGRAM_VECTOR:
-#pragma unroll
-                    for (int k = 0; k < NV; ++k) if (idx == (uint32_t)k) out = v[k];
-                    break;
-                default:
-                    out = L::splat(p.imm[idx & (MI355X_PROGRAM_MAX_IMM - 1)]);
+                case MI355X_PROGRAM_REG: MI355X_PICK(r, NR) break;
+                case MI355X_PROGRAM_TENSOR: MI355X_PICK(t, NT) break;
+                case MI355X_PROGRAM_VECTOR: MI355X_PICK(v, NV) break;
+                default: out = L::splat(p.imm[idx & (MI355X_PROGRAM_MAX_IMM - 1)]);
             }
+#undef MI355X_PICK
             return out;
         };
         V result = L::splat(0.f);
@@ -121,7 +117,7 @@ __global__ __launch_bounds__(256) void eltwise_program_kernel(ProgramArgs p) {
             result = program_op<V>((int)(ins & 255u), fetch((ins >> 16) & 255u), fetch(ins >> 24));
             const uint32_t dst = (ins >> 8) & 255u;
 #pragma unroll
-            for (int k = 0; k < NR; ++k) if (dst == (uint32_t)k) r[k] = result;   // uniform
+            for (int k = 0; k < NR; ++k) if (dst == (uint32_t)k) { r[k] = result; asm volatile(""); }   // uniform
         }
         __builtin_nontemporal_store(result, reinterpret_cast<V*>(p.Y) + i);
     }
