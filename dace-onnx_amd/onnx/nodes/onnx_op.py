@@ -7,9 +7,8 @@ import itertools
 import logging
 import typing
 
-from ... import sdfg as dace
 from ...sdfg import SDFG, SDFGState, LibraryNode, MultiConnectorEdge
-from ..schema import ONNXSchema, ONNXParameterType, ONNXAttributeType, SCHEMAS
+from ..schema import ONNXSchema, ONNXParameterType, SCHEMAS
 from .node_utils import parse_variadic_param
 
 log = logging.getLogger(__name__)

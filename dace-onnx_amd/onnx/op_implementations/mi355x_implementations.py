@@ -38,8 +38,6 @@ call, so an unsupported configuration is refused before anything is launched
 (and, there being no ONNX Runtime here, reported as an error by the fallback).
 ``forward`` returns a :class:`~dace_onnx_amd.sdfg.KernelCall`.
 """
-import typing
-
 import numpy as np
 
 from ... import sdfg as dace

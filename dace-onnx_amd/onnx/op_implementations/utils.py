@@ -1,6 +1,5 @@
 """Helpers for writing expansions (``daceml/onnx/op_implementations/utils.py``)."""
 import copy
-import typing
 
 from ... import sdfg as dace
 from ...sdfg import SDFG, SDFGState

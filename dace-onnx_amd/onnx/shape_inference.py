@@ -11,7 +11,7 @@ import typing
 
 import numpy as np
 
-from .proto import ModelProto, ValueInfoProto, TensorProto, np_dtype_to_tensor_dtype
+from .proto import ModelProto, ValueInfoProto, TensorProto
 
 
 class ShapeInferenceError(ValueError):

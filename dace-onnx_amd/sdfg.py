@@ -22,8 +22,6 @@ arguments are staged in and out, and there is no host implementation of any
 node; a library node that was not expanded to kernels cannot run.
 """
 import collections
-import copy
-import ctypes
 import itertools
 import typing
 

@@ -4,7 +4,7 @@ import functools
 import logging
 import typing
 
-from ..sdfg import SDFG, SDFGState, Node, MultiConnectorEdge, Array, NestedSDFG, LibraryNode
+from ..sdfg import SDFG, SDFGState, Node, MultiConnectorEdge, Array, NestedSDFG
 
 log = logging.getLogger(__name__)
 
