@@ -15,6 +15,7 @@ uploaded once at construction.
 import collections
 import logging
 import re
+import copy
 import typing
 from itertools import chain, repeat
 
@@ -109,6 +110,7 @@ class ONNXModel:
         if fold_constants:
             from ..transformation.constant_folding import fold_constants as _fold
             model = _fold(model)
+        model = self._separate_passthrough_outputs(model)
         for node in model.graph.node:
             if not has_onnx_node(node.op_type):
                 raise ValueError("Unsupported ONNX operator: '{}'".format(node.op_type))
@@ -240,6 +242,32 @@ class ONNXModel:
             extra.append(proto.numpy_helper.from_array(value, name=node.output[0]))
         model.graph.node = kept
         model.graph.initializer = list(model.graph.initializer) + extra
+        return model
+
+    @staticmethod
+    def _separate_passthrough_outputs(model: ModelProto) -> ModelProto:
+        """A graph output that is a graph input or an initializer itself (legal ONNX; also what remains when
+        constant folding consumes every node) gets an ``Identity`` node and a name of its own, so that the
+        caller's output buffer and the input are two arrays. The caller's model is not modified."""
+        graph = model.graph
+        sources = {v.name for v in graph.input} | {t.name for t in graph.initializer}
+        if not any(o.name in sources for o in graph.output):
+            return model
+        model = copy.copy(model)
+        model.graph = graph = copy.copy(graph)
+        taken = sources | {o for n in graph.node for o in n.output}
+        graph.node, graph.output = list(graph.node), list(graph.output)
+        for i, out in enumerate(graph.output):
+            if out.name not in sources:
+                continue
+            new_name = out.name + "_output"
+            while new_name in taken:
+                new_name += "_"
+            taken.add(new_name)
+            graph.node.append(proto.helper.make_node("Identity", [out.name], [new_name], name="passthrough_" + new_name))
+            renamed = copy.copy(out)
+            renamed.name = new_name
+            graph.output[i] = renamed
         return model
 
     @staticmethod

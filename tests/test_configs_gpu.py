@@ -489,3 +489,22 @@ def test_tasklet_fusion_programs_values():
     for name, (m, inputs, fn) in _tasklet_fusion_graphs().items():
         result = donnx.ONNXModel("tf_values_" + name, m)(*([A, B][:len(inputs)]))
         assert np.allclose(result, fn(A, B)), name
+
+
+def test_outputs_that_are_inputs_or_weights():
+    # a graph output may be a graph input or an initializer itself: each comes back as a copy in a buffer of its own
+    H, T = proto.helper, proto.TensorProto
+    g = H.make_graph([H.make_node("Relu", ["x"], ["r"])], "g", [H.make_tensor_value_info("x", T.FLOAT, [2, 3])],
+                     [H.make_tensor_value_info("x", T.FLOAT, [2, 3]), H.make_tensor_value_info("r", T.FLOAT, [2, 3]),
+                      H.make_tensor_value_info("w", T.FLOAT, [3])],
+                     initializer=[proto.numpy_helper.from_array(np.arange(3, dtype=np.float32), "w")])
+    model = donnx.ONNXModel("passthrough", H.make_model(g, opset_imports=[H.make_opsetid("", 12)]))
+    x = np.random.default_rng(13).normal(size=(2, 3)).astype(np.float32)
+    same, relu, w = model(x)
+    assert np.array_equal(same, x) and np.array_equal(relu, np.maximum(x, 0)) and np.array_equal(w, np.arange(3, dtype=np.float32))
+    xt = torch.from_numpy(x).cuda()
+    same_t, _, _ = model(xt)
+    assert same_t.data_ptr() != xt.data_ptr() and torch.equal(same_t, xt)
+    # the model with no node at all
+    g0 = H.make_graph([], "g0", [H.make_tensor_value_info("x", T.FLOAT, [2, 3])], [H.make_tensor_value_info("x", T.FLOAT, [2, 3])])
+    assert np.array_equal(donnx.ONNXModel("empty", H.make_model(g0, opset_imports=[H.make_opsetid("", 12)]))(x), x)
