@@ -508,3 +508,42 @@ def test_outputs_that_are_inputs_or_weights():
     # the model with no node at all
     g0 = H.make_graph([], "g0", [H.make_tensor_value_info("x", T.FLOAT, [2, 3])], [H.make_tensor_value_info("x", T.FLOAT, [2, 3])])
     assert np.array_equal(donnx.ONNXModel("empty", H.make_model(g0, opset_imports=[H.make_opsetid("", 12)]))(x), x)
+
+
+def test_conv_network_hip_graph_replays_match_eager():
+    """A convolution network (Conv+BatchNormalization+Relu folded, MaxPool through LDS, residual epilogue, global
+    average pooling, Gemm, LogSoftmax) replayed as one HIP graph: every replay, with eager work and synchronisation
+    in between and changing inputs, equals the eager result bit for bit."""
+    H, T = proto.helper, proto.TensorProto
+    rng = np.random.default_rng(14)
+    f32 = lambda *s: rng.normal(size=s).astype(np.float32)
+    inits = {"w1": f32(16, 3, 3, 3) * 0.2, "b1": f32(16), "s1": f32(16), "be1": f32(16), "m1": f32(16),
+             "v1": rng.uniform(0.5, 2.0, size=16).astype(np.float32), "w2": f32(16, 16, 3, 3) * 0.1, "wf": f32(10, 16), "bf": f32(10)}
+    nodes = [H.make_node("Conv", ["x", "w1", "b1"], ["c1"], pads=[1, 1, 1, 1]),
+             H.make_node("BatchNormalization", ["c1", "s1", "be1", "m1", "v1"], ["n1"]), H.make_node("Relu", ["n1"], ["r1"]),
+             H.make_node("MaxPool", ["r1"], ["p1"], kernel_shape=[3, 3], strides=[2, 2], pads=[1, 1, 1, 1]),
+             H.make_node("Conv", ["p1", "w2"], ["c2"], pads=[1, 1, 1, 1]), H.make_node("Add", ["c2", "p1"], ["a2"]),
+             H.make_node("Relu", ["a2"], ["r2"]), H.make_node("GlobalAveragePool", ["r2"], ["g"]),
+             H.make_node("Flatten", ["g"], ["f"], axis=1), H.make_node("Gemm", ["f", "wf", "bf"], ["l"], transB=1),
+             H.make_node("LogSoftmax", ["l"], ["y"], axis=1)]
+    g = H.make_graph(nodes, "cnn", [H.make_tensor_value_info("x", T.FLOAT, [8, 3, 64, 64])],
+                     [H.make_tensor_value_info("y", T.FLOAT, [8, 10])],
+                     initializer=[proto.numpy_helper.from_array(v, k) for k, v in inits.items()])
+    m = H.make_model(g, opset_imports=[H.make_opsetid("", 12)])
+    model = donnx.ONNXModel("cnn_graph", m, use_hip_graph=True)
+    assert model.compile_and_init().num_launches == 6     # conv, maxpool, conv + residual + relu, mean, gemm, logsoftmax
+    xs = [torch.from_numpy(f32(8, 3, 64, 64)).cuda() for _ in range(3)]
+    model(xs[0])                                          # first call runs eagerly and captures
+    for i in range(5):
+        xi = xs[i % 3]
+        replayed = model(xi).clone()
+        torch.cuda.synchronize()
+        ref = donnx.ONNXModel(f"cnn_eager_{i}", m)(xi)
+        assert torch.equal(replayed, ref), i
+    # and the values: against the oracle, node by node
+    x = xs[1].cpu().numpy()
+    r1 = O.relu(O.batch_normalization(O.conv2d(x, inits["w1"], inits["b1"], pads=(1, 1, 1, 1)), inits["s1"], inits["be1"], inits["m1"], inits["v1"]))
+    p1 = O.maxpool2d(r1, (3, 3), (2, 2), (1, 1, 1, 1))
+    r2 = O.relu(O.conv2d(p1, inits["w2"], None, pads=(1, 1, 1, 1)) + p1)
+    logits = O.gemm(O.global_average_pool(r2).reshape(8, 16), inits["wf"], inits["bf"], transB=1)
+    assert rel_err(O.log_softmax(logits, axis=1), model(xs[1]).cpu().numpy()) < FP32_REL_TOL
