@@ -273,6 +273,53 @@ def test_transformation_test_modules_results(cls, shape, launches):
     torch_tensors_close("output", torch_module(input), dace_module(input.cuda()).cpu())
 
 
+class _TwoConvs(nn.Module):
+    """tests/pytorch/test_conv2d.py:12-21 of the reference."""
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(1, 4, 3)
+        self.conv2 = nn.Conv2d(4, 4, 3)
+
+    def forward(self, x):
+        x = torch.relu(self.conv1(x))
+        return torch.relu(self.conv2(x))
+
+
+@pytest.mark.gpu
+def test_conv2d_wrapped_and_decorated(sdfg_name):
+    # tests/pytorch/test_conv2d.py:11-38
+    torch.manual_seed(9)
+    ptmodel = _TwoConvs()
+    x = torch.rand(1, 1, 8, 8)
+
+    @dace_module(sdfg_name=sdfg_name)
+    class TestDecorator(_TwoConvs):
+        pass
+
+    dace_model = DaceModule(ptmodel, sdfg_name=sdfg_name + "_wrapped")
+    dace_output = dace_model(x.cuda())
+    decorated = TestDecorator()
+    decorated_output = decorated(x.cuda())
+    assert np.allclose(ptmodel(x).detach().numpy(), dace_output.cpu().numpy(), atol=1e-06)
+    assert np.allclose(decorated.model(x).detach().numpy(), decorated_output.cpu().numpy(), atol=1e-06)
+
+
+@pytest.mark.gpu
+def test_debug_transients_decorator():
+    # tests/pytorch/test_debug_transients.py:8-23: the intermediate comes back as a second output
+    @dace_module(debug_transients=True)
+    class Module(nn.Module):
+        def forward(self, x):
+            y = x + 3
+            return y * 5
+
+    module = Module()
+    x = torch.rand(5, 5)
+    output, y = module(x.cuda())
+    torch_tensors_close("output", (x + 3) * 5, output.cpu())
+    torch_tensors_close("y", x + 3, y.cpu())
+
+
 class _LogSqrt(nn.Module):
     """The example of the reference's DaceModule docstring (daceml/pytorch/module.py:43-55)."""
     def forward(self, x):
