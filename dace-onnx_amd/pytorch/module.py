@@ -267,6 +267,8 @@ class DaceModule(nn.Module):
     :param training: must be False (the graph is the inference graph).
     :param backward: must be False.
     :param auto_optimize: apply the graph-level fusion pass (registered as the post-ONNX hook "auto_optimize").
+    :param use_hip_graph: replay the launch sequence as one HIP graph from the second call on (inputs are copied
+                          into the graph's buffers; not in the reference, whose launches go through DaCe's streams).
     :param debug_transients: every intermediate value becomes an additional output of the module (a post-ONNX
                              hook placed before the optimisation, so nothing is fused across them).
     :param sdfg_name: the name to give to the SDFG (defaults to the module's class name).
@@ -279,8 +281,9 @@ class DaceModule(nn.Module):
     def __init__(self, module: nn.Module, dummy_inputs: typing.Optional[typing.Tuple[torch.Tensor]] = None,
                  cuda: typing.Optional[bool] = None, training: bool = False, backward=False, apply_strict: bool = True,
                  auto_optimize: bool = True, debug_transients: bool = False, sdfg_name: typing.Optional[str] = None,
-                 exporter: str = "auto"):
+                 exporter: str = "auto", use_hip_graph: bool = False):
         super().__init__()
+        self.use_hip_graph = use_hip_graph
         if exporter not in ("auto", "structural", "torch"):
             raise ValueError(f"exporter must be 'auto', 'structural' or 'torch', got {exporter!r}")
         self.exporter = exporter
@@ -371,7 +374,7 @@ class DaceModule(nn.Module):
             self.model.train(was_training)
         # optimisation is a hook of this module, not of the ONNXModel (which would apply it on its first call)
         self.dace_model = ONNXModel(self.sdfg_name, self.onnx_model, cuda=True, parent_pytorch_module=self.model,
-                                    auto_optimize=False)
+                                    auto_optimize=False, use_hip_graph=self.use_hip_graph)
         self.sdfg = self.dace_model.sdfg
         for hook in self.post_onnx_hooks.values():
             hook(self)

@@ -174,6 +174,17 @@ def test_lenet_launch_list():
 
 
 @pytest.mark.gpu
+def test_lenet_hip_graph_replay(sdfg_name):
+    torch.manual_seed(10)
+    net = _LeNet()
+    dace_net = DaceModule(copy.deepcopy(net), sdfg_name=sdfg_name, use_hip_graph=True)
+    for i in range(4):        # the first call runs eagerly and captures, the others replay
+        input = torch.rand(8, 1, 32, 32)
+        torch_tensors_close(f"output_{i}", net(input), dace_net(input.cuda()).cpu())
+        torch.cuda.synchronize()
+
+
+@pytest.mark.gpu
 def test_lenet(sdfg_name):
     # tests/pytorch/test_lenet.py:37-57
     torch.manual_seed(7)
