@@ -44,6 +44,7 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
                                  _c_i64_p, _c_i64_p, _c_i64_p, _int, _vp]),
     "mi355x_conv2d_res_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                      _c_i64_p, _c_i64_p, _c_i64_p, _int, _vp]),
+    "mi355x_matmul_integer": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _i64, _i64, _vp]),
     "mi355x_matmul_integer_i8": (_int, [_vp, _vp, _vp, _vp, _vp,
                                         _i64, _i64, _i64, _vp]),
     "mi355x_softmax_f32": (_int, [_vp, _vp, _i64, _i64, _i64, _vp]),

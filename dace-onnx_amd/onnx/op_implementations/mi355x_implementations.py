@@ -549,35 +549,54 @@ class MI355XBatchNormalization(ONNXForward):
 
 @op_implementation(op="MatMulInteger", name=IMPLEMENTATION_NAME)
 class MI355XMatMulInteger(ONNXForward):
-    """int8 x int8 -> int32 on int8 MFMA, bit-exact, scalar zero points read on
-    the device. The reference can only run this node through ONNX Runtime."""
+    """8-bit x 8-bit -> int32 on int8 MFMA, bit-exact; operands int8 or uint8 (independently), zero
+    points read on the device: absent, one value, one per row of A or one per column of B. A may be
+    a stack of matrices against a 2-D B (the stack is folded into M). The reference can only run this
+    node through ONNX Runtime (onnx_op.py:686-687)."""
 
     @staticmethod
-    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+    def _plan(node, state, sdfg):
         A = in_desc_with_name(node, state, sdfg, "A")
         B = in_desc_with_name(node, state, sdfg, "B")
         Y = out_desc_with_name(node, state, sdfg, "Y")
-        if A.dtype != dace.int8 or B.dtype != dace.int8 or Y.dtype != dace.int32:
-            return False
-        if len(A.shape) != 2 or len(B.shape) != 2 or A.shape[1] != B.shape[0]:
-            return False
-        if tuple(Y.shape) != (A.shape[0], B.shape[1]) or not _contig(A, B, Y):
-            return False
-        for zp in ("a_zero_point", "b_zero_point"):
-            if _has_input(node, state, zp):
-                d = in_desc_with_name(node, state, sdfg, zp)
-                if d.dtype != dace.int8 or d.total_size != 1:  # per-row / per-column zero points
-                    return False
-        return True
+        eight_bit = (dace.int8, dace.uint8)
+        if A.dtype not in eight_bit or B.dtype not in eight_bit or Y.dtype != dace.int32:
+            return None
+        if len(A.shape) < 2 or len(B.shape) != 2 or A.shape[-1] != B.shape[0]:
+            return None
+        M, K, N = prod(A.shape[:-1]), A.shape[-1], B.shape[1]
+        if tuple(Y.shape) != tuple(A.shape[:-1]) + (N, ) or not _contig(A, B, Y):
+            return None
+        counts = {}
+        for zp, operand, full in (("a_zero_point", A, M), ("b_zero_point", B, N)):
+            counts[zp] = 1
+            if not _has_input(node, state, zp):
+                continue
+            d = in_desc_with_name(node, state, sdfg, zp)
+            if d.dtype != operand.dtype or not _contig(d):
+                return None
+            if d.total_size == 1:
+                continue
+            # one per row of A: [M] for a matrix, [D1, ..., M, 1] for a stack; one per column of B: [N]
+            shape = tuple(d.shape)
+            per_row = shape == (A.shape[0], ) if len(A.shape) == 2 else shape == tuple(A.shape[:-1]) + (1, )
+            if not (per_row if zp == "a_zero_point" else shape == (N, )):
+                return None
+            counts[zp] = full
+        return M, N, K, A.dtype == dace.uint8, B.dtype == dace.uint8, counts["a_zero_point"], counts["b_zero_point"]
+
+    @staticmethod
+    def forward_can_be_applied(node, state: SDFGState, sdfg: SDFG) -> bool:
+        return MI355XMatMulInteger._plan(node, state, sdfg) is not None
 
     @staticmethod
     def forward(node, state: SDFGState, sdfg: SDFG):
-        A = in_desc_with_name(node, state, sdfg, "A")
-        B = in_desc_with_name(node, state, sdfg, "B")
+        M, N, K, a_unsigned, b_unsigned, za_count, zb_count = MI355XMatMulInteger._plan(node, state, sdfg)
         za = "a_zero_point" if _has_input(node, state, "a_zero_point") else None
         zb = "b_zero_point" if _has_input(node, state, "b_zero_point") else None
-        return kernel_call_for_node(node, state, "mi355x_matmul_integer_i8", [
-            Ptr("A"), Ptr("B"), Ptr(za), Ptr(zb), Ptr("Y"), A.shape[0], B.shape[1], A.shape[1], Stream()])
+        return kernel_call_for_node(node, state, "mi355x_matmul_integer", [
+            Ptr("A"), Ptr("B"), Ptr(za), Ptr(zb), Ptr("Y"), M, N, K, int(a_unsigned), int(b_unsigned), za_count, zb_count,
+            Stream()])
 
 
 # ------------------------------------------------------------------------------------

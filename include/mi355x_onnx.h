@@ -134,14 +134,26 @@ int mi355x_batchnorm_f32(const float* X, const float* scale, const float* B, con
                          const float* var, float* Y, int64_t N, int64_t C, int64_t HW, float eps,
                          void* stream);
 
-/* ONNX MatMulInteger, int8 x int8 -> int32 on int8 MFMA, bit-exact.
- *   Y[m,n] = sum_k (A[m,k] - a_zero_point) * (B[k,n] - b_zero_point)
+/* ONNX MatMulInteger (opset 10), 8-bit operands -> int32 on int8 MFMA, bit-exact.
+ *   Y[m,n] = sum_k (A[m,k] - a_zero_point[m]) * (B[k,n] - b_zero_point[n])
  * The reference has no expansion of its own for this node: the generated class
- * (daceml/onnx/nodes/onnx_op.py:623-640) only has the "onnxruntime"
- * implementation (onnx_op.py:686-687 -> node_codegen.py:321-573).
- * A is [M,K], B is [K,N], Y is [M,N], all C-contiguous. The zero points are
- * the node's optional scalar inputs: DEVICE pointers to one int8 each, read by
- * the kernel (no host synchronisation); NULL means 0. */
+ * (daceml/onnx/nodes/onnx_op.py:623-640, built from the ONNX schema: T1, T2 in
+ * {int8, uint8}, optional zero points of the operand's type) only has the
+ * "onnxruntime" implementation (onnx_op.py:686-687 -> node_codegen.py:321-573).
+ * A is [M,K], B is [K,N], Y is [M,N], all C-contiguous; a stack of A matrices
+ * against one B is the same call with the stack folded into M.
+ * a_unsigned / b_unsigned: the operand (and its zero point) is uint8, else int8.
+ * The zero points are DEVICE pointers read by the kernel (no host
+ * synchronisation); NULL means 0. a_zero_point_count is 1 (one value) or M (one
+ * per row of A), b_zero_point_count is 1 or N (one per column of B). */
+int mi355x_matmul_integer(const void* A, const void* B,
+                          const void* a_zero_point, const void* b_zero_point,
+                          int32_t* Y, int64_t M, int64_t N, int64_t K,
+                          int a_unsigned, int b_unsigned,
+                          int64_t a_zero_point_count, int64_t b_zero_point_count,
+                          void* stream);
+
+/* The same with int8 operands and one zero point each (or NULL). */
 int mi355x_matmul_integer_i8(const int8_t* A, const int8_t* B,
                              const int8_t* a_zero_point, const int8_t* b_zero_point,
                              int32_t* Y, int64_t M, int64_t N, int64_t K,

@@ -72,10 +72,17 @@ def gelu(X):
 
 
 def matmul_integer(A, B, a_zero_point=0, b_zero_point=0):
-    A, B = np.ascontiguousarray(A, np.int8), np.ascontiguousarray(B, np.int8)
-    Y = np.empty((A.shape[0], B.shape[1]), np.int32)
-    library().oracle_matmul_integer_i8(_p(A), _p(B), ctypes.c_int32(int(a_zero_point)), ctypes.c_int32(int(b_zero_point)),
-                                       _p(Y), *[ctypes.c_int64(v) for v in (A.shape[0], B.shape[1], A.shape[1])])
+    """int8 / uint8 operands (2-D), zero points scalar, per row of A ([M]) or per column of B ([N])."""
+    A, B = np.ascontiguousarray(A), np.ascontiguousarray(B)
+    assert A.dtype in (np.int8, np.uint8) and B.dtype in (np.int8, np.uint8) and A.ndim == 2 and B.ndim == 2
+    M, K, N = A.shape[0], A.shape[1], B.shape[1]
+    za = np.ascontiguousarray(np.asarray(a_zero_point).reshape(-1), np.int32)
+    zb = np.ascontiguousarray(np.asarray(b_zero_point).reshape(-1), np.int32)
+    assert za.size in (1, M) and zb.size in (1, N)
+    Y = np.empty((M, N), np.int32)
+    library().oracle_matmul_integer(_p(A), _p(B), _p(za), _p(zb), _p(Y), *[ctypes.c_int64(v) for v in (M, N, K)],
+                                    ctypes.c_int(A.dtype == np.uint8), ctypes.c_int(B.dtype == np.uint8),
+                                    ctypes.c_int64(0 if za.size == 1 else 1), ctypes.c_int64(0 if zb.size == 1 else 1))
     return Y
 
 

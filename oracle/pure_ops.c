@@ -139,6 +139,30 @@ void oracle_matmul_integer_i8(const int8_t* A, const int8_t* B, int32_t za, int3
     }
 }
 
+/* The same for int8 or uint8 operands and zero points given per row of A (za_stride 1) and per column
+ * of B (zb_stride 1) or as one value (stride 0); int32 accumulation wraps modulo 2^32 like the node's
+ * int32 output. */
+void oracle_matmul_integer(const void* A, const void* B, const int32_t* za, const int32_t* zb, int32_t* Y,
+                           int64_t M, int64_t N, int64_t K, int a_unsigned, int b_unsigned,
+                           int64_t za_stride, int64_t zb_stride) {
+    const int8_t* As = (const int8_t*)A;
+    const uint8_t* Au = (const uint8_t*)A;
+    const int8_t* Bs = (const int8_t*)B;
+    const uint8_t* Bu = (const uint8_t*)B;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        uint32_t* y = (uint32_t*)&Y[m * N];
+        memset(y, 0, sizeof(int32_t) * (size_t)N);
+        for (int64_t k = 0; k < K; ++k) {
+            const int32_t a = (a_unsigned ? (int32_t)Au[m * K + k] : (int32_t)As[m * K + k]) - za[m * za_stride];
+            for (int64_t n = 0; n < N; ++n) {
+                const int32_t b = (b_unsigned ? (int32_t)Bu[k * N + n] : (int32_t)Bs[k * N + n]) - zb[n * zb_stride];
+                y[n] += (uint32_t)(a * b);
+            }
+        }
+    }
+}
+
 /* MatMul without a BLAS library: DaCe's pure map-reduce GEMM, what
  * create_einsum_sdfg falls back to (pure_implementations.py:260-266). */
 void oracle_matmul_f32(const float* A, const float* B, float* Y, int64_t M, int64_t N, int64_t K) {

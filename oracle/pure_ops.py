@@ -81,11 +81,17 @@ def gemm(A, B, C=None, alpha=1.0, beta=1.0, transA=0, transB=0):
 
 def matmul_integer(A, B, a_zero_point=0, b_zero_point=0):
     """ONNX MatMulInteger (opset 10): ``(A - a_zp) @ (B - b_zp)`` accumulated in
-    int32. The reference expands this node only through ONNX Runtime
-    (onnx_op.py:686-687); this is the specification's formula, evaluated in int64
-    and wrapped to int32."""
-    a = A.astype(np.int64) - np.int64(a_zero_point)
-    b = B.astype(np.int64) - np.int64(b_zero_point)
+    int32, operands int8 or uint8. ``a_zero_point`` is one value or one per row of
+    A (``[M]`` for a matrix, ``[..., M, 1]`` for a stack), ``b_zero_point`` one
+    value or one per column of B (``[N]``). The reference expands this node only
+    through ONNX Runtime (onnx_op.py:686-687); this is the specification's formula,
+    evaluated in int64 and wrapped to int32."""
+    a_zp = np.asarray(a_zero_point).astype(np.int64)
+    if a_zp.ndim == 1 and a_zp.size > 1:
+        a_zp = a_zp.reshape(-1, 1)
+    b_zp = np.asarray(b_zero_point).astype(np.int64)
+    a = A.astype(np.int64) - a_zp
+    b = B.astype(np.int64) - b_zp
     return (a @ b).astype(np.int32)
 
 

@@ -152,7 +152,7 @@ def test_validate_errors():
         sdfg.expand_library_nodes()
 
 
-@pytest.mark.parametrize("case", ["matmul_1d", "conv_group", "conv_3d", "mmi_per_row_zp", "gelu_tanh", "ln_mean_out",
+@pytest.mark.parametrize("case", ["matmul_1d", "conv_group", "conv_3d", "mmi_zp_wrong_length", "gelu_tanh", "ln_mean_out",
                                   "softmax_f64", "gemm_beta"])
 def test_refusal_is_an_error_not_a_fallback(case):
     """forward_can_be_applied -> False falls back to "onnxruntime" (onnx_op.py:668-680), which this
@@ -166,9 +166,9 @@ def test_refusal_is_an_error_not_a_fallback(case):
     elif case == "conv_3d":
         sdfg, _ = _one_node_sdfg(donnx.ONNXConv("c"), {"X": ([1, 2, 8, 8, 8], f32), "W": ([4, 2, 3, 3, 3], f32)},
                                  {"Y": ([1, 4, 6, 6, 6], f32)})
-    elif case == "mmi_per_row_zp":
+    elif case == "mmi_zp_wrong_length":
         sdfg, _ = _one_node_sdfg(donnx.ONNXMatMulInteger("m"),
-                                 {"A": ([4, 8], i8), "B": ([8, 4], i8), "a_zero_point": ([4], i8)}, {"Y": ([4, 4], i32)})
+                                 {"A": ([4, 8], i8), "B": ([8, 4], i8), "a_zero_point": ([3], i8)}, {"Y": ([4, 4], i32)})
     elif case == "gelu_tanh":
         sdfg, _ = _one_node_sdfg(donnx.ONNXGelu("g", approximate="tanh"), {"X": ([4], f32)}, {"Y": ([4], f32)})
     elif case == "ln_mean_out":

@@ -712,7 +712,9 @@ def test_reshape_is_a_view_inside_a_graph():
 @pytest.mark.parametrize("M, N, K, za, zb", [(128, 128, 64, 0, 0), (128, 128, 64, 3, -2), (512, 384, 768, 3, -2),
                                              (100, 52, 37, 5, 7), (130, 260, 48, -128, 127), (1, 1, 1, 1, 1),
                                              (33, 2, 16, 0, 9), (7, 129, 1000, -7, 0),
-                                             # K % 128 == 0 and N % 4 == 0: the pipelined kernel, ragged M and N tiles
+                                             # K % 64 == 0 and N % 16 == 0: the pipelined kernel, ragged M and N tiles
+                                             (200, 144, 256, 3, -2), (1, 16, 128, -128, 127), (257, 400, 640, 0, 11),
+                                             (129, 112, 1152, -9, 0), (130, 272, 64, 5, 5),
                                              (128, 128, 128, 0, 0), (200, 132, 256, 3, -2), (1, 4, 128, -128, 127),
                                              (257, 388, 640, 0, 11), (129, 124, 1152, -9, 0), (384, 256, 384, 1, 1)])
 def test_matmul_integer_bit_exact(M, N, K, za, zb):
@@ -732,6 +734,61 @@ def test_matmul_integer_without_zero_points_and_extremes():
     assert np.all(Y == 768 * 128 * 128)
     donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array([127], np.int8), b_zero_point=np.array([127], np.int8), Y=Y)
     assert np.all(Y == 768 * 255 * 255)
+
+
+@pytest.mark.parametrize("a_dt, b_dt", [(np.uint8, np.int8), (np.int8, np.uint8), (np.uint8, np.uint8)])
+@pytest.mark.parametrize("M, N, K", [(256, 256, 128), (200, 144, 192), (100, 52, 37), (384, 256, 64), (1, 16, 64)])
+def test_matmul_integer_unsigned_operands_bit_exact(a_dt, b_dt, M, N, K):
+    """uint8 operands (ONNX MatMulInteger T1 / T2, the node class of onnx_op.py:623-640): scalar zero points of the
+    operand's type, no zero points, against the integer formula. Parity unpinned against the reference itself,
+    which runs the node only inside ONNX Runtime."""
+    rng = np.random.default_rng(31)
+    A = rng.integers(0, 256, size=(M, K)).astype(a_dt) if a_dt == np.uint8 else rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(0, 256, size=(K, N)).astype(b_dt) if b_dt == np.uint8 else rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    za, zb = np.array(131 if a_dt == np.uint8 else -3, a_dt), np.array(250 if b_dt == np.uint8 else 7, b_dt)
+    Y = np.zeros((M, N), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=za, b_zero_point=zb, Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B, za, zb), Y)
+    donnx.ONNXMatMulInteger(A=A, B=B, Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B), Y)
+    donnx.ONNXMatMulInteger(A=A, B=B, b_zero_point=zb, Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B, 0, zb), Y)
+
+
+@pytest.mark.parametrize("M, N, K", [(256, 256, 128), (130, 80, 64), (77, 36, 50)])
+def test_matmul_integer_zero_point_per_row_and_column(M, N, K):
+    rng = np.random.default_rng(32)
+    A = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    za = rng.integers(0, 256, size=M).astype(np.uint8)
+    zb = rng.integers(-128, 128, size=N, dtype=np.int8)
+    Y = np.zeros((M, N), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=za, b_zero_point=zb, Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B, za, zb), Y)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=za, Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B, za, 0), Y)
+
+
+def test_matmul_integer_stack_of_matrices():
+    rng = np.random.default_rng(33)
+    A = rng.integers(-128, 128, size=(3, 64, 128), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(128, 48), dtype=np.int8)
+    za = rng.integers(-128, 128, size=(3, 64, 1), dtype=np.int8)
+    Y = np.zeros((3, 64, 48), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=za, b_zero_point=np.array(-2, np.int8), Y=Y)
+    assert np.array_equal(O.matmul_integer(A, B, za, -2), Y)
+
+
+def test_matmul_integer_several_tiles_per_workgroup():
+    """More 128 x 128 tiles than resident workgroups: a workgroup stores one tile while it multiplies the next."""
+    rng = np.random.default_rng(34)
+    M, N, K = 4096, 4096, 128
+    A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    Y = np.zeros((M, N), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array(3, np.int8), b_zero_point=np.array(-2, np.int8), Y=Y)
+    ref = (A.astype(np.int32) - 3) @ (B.astype(np.int32) + 2)
+    assert np.array_equal(ref, Y)
 
 
 # ----------------------------------------------------------------------------- edge cases

@@ -322,6 +322,49 @@ def test_matmul_integer_identity_and_extremes():
     assert not np.array_equal(y, O.matmul_integer(A, B, zb, za))
 
 
+def test_matmul_integer_unsigned_operands_and_zero_point_vectors(c_oracle):
+    """uint8 operands and one zero point per row of A / per column of B (ONNX MatMulInteger, T1 and T2 in
+    {int8, uint8}): brute force in Python integers, the row/column-sum identity, and the case that must
+    reduce to the signed one (u - 128 as int8 with the zero point moved by 128)."""
+    rng = np.random.default_rng(21)
+    M, K, N = 9, 37, 11
+    for a_dt, b_dt in ((np.uint8, np.int8), (np.int8, np.uint8), (np.uint8, np.uint8)):
+        lo_a, hi_a = (0, 256) if a_dt == np.uint8 else (-128, 128)
+        lo_b, hi_b = (0, 256) if b_dt == np.uint8 else (-128, 128)
+        A = rng.integers(lo_a, hi_a, size=(M, K)).astype(a_dt)
+        B = rng.integers(lo_b, hi_b, size=(K, N)).astype(b_dt)
+        za = rng.integers(lo_a, hi_a, size=M).astype(a_dt)
+        zb = rng.integers(lo_b, hi_b, size=N).astype(b_dt)
+        y = O.matmul_integer(A, B, za, zb)
+        brute = [[sum((int(A[m, k]) - int(za[m])) * (int(B[k, n]) - int(zb[n])) for k in range(K)) for n in range(N)]
+                 for m in range(M)]
+        assert np.array_equal(y, np.array(brute, dtype=np.int64).astype(np.int32))
+        assert np.array_equal(y, c_oracle.matmul_integer(A, B, za, zb))
+        a64, b64, za64, zb64 = A.astype(np.int64), B.astype(np.int64), za.astype(np.int64)[:, None], zb.astype(np.int64)[None, :]
+        ident = a64 @ b64 - zb64 * a64.sum(1, keepdims=True) - za64 * b64.sum(0, keepdims=True) + K * za64 * zb64
+        assert np.array_equal(y, ident.astype(np.int32))
+        # scalar zero points of the operand's type
+        ys = O.matmul_integer(A, B, za[0], zb[0])
+        assert np.array_equal(ys, c_oracle.matmul_integer(A, B, za[0], zb[0]))
+        assert np.array_equal(ys[0], y[0] if N == 1 else np.array([sum((int(A[0, k]) - int(za[0])) * (int(B[k, n]) - int(zb[0]))
+                                                                      for k in range(K)) for n in range(N)], dtype=np.int32))
+    # reduction to the signed case
+    Au = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    Bs = rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+    As = (Au.astype(np.int16) - 128).astype(np.int8)
+    assert np.array_equal(O.matmul_integer(Au, Bs, np.uint8(200), np.int8(-5)), O.matmul_integer(As, Bs, np.int8(72), np.int8(-5)))
+    # extreme values: (255 - 0) * (255 - 0) * K and (0 - 255)(255 - 0) K stay inside int32 for K = 768
+    Ae, Be = np.full((2, 768), 255, np.uint8), np.full((768, 2), 255, np.uint8)
+    assert np.all(O.matmul_integer(Ae, Be) == 768 * 255 * 255)
+    assert np.all(O.matmul_integer(np.zeros_like(Ae), Be, np.uint8(255), np.uint8(0)) == -768 * 255 * 255)
+    # a stack of matrices with a per-row zero point of shape [D, M, 1]
+    A3 = rng.integers(0, 256, size=(2, M, K)).astype(np.uint8)
+    z3 = rng.integers(0, 256, size=(2, M, 1)).astype(np.uint8)
+    y3 = O.matmul_integer(A3, Bs, z3, np.int8(4))
+    for d in range(2):
+        assert np.array_equal(y3[d], O.matmul_integer(A3[d], Bs, z3[d, :, 0], np.int8(4)))
+
+
 # ----------------------------------------------------------------------------- C restatement vs numpy restatement
 def test_c_oracle_matches_numpy_oracle(c_oracle):
     rng = np.random.default_rng(11)
