@@ -3,30 +3,37 @@ construction, validation and implementation-binding behaviour
 (``daceml/onnx/nodes/onnx_op.py:84-415`` ONNXOp and validate, ``:494-694`` class
 generation and binding, ``:418-475`` the Python-frontend call form).
 """
-import itertools
 import logging
 import typing
 
 from ...sdfg import SDFG, SDFGState, LibraryNode, MultiConnectorEdge
-from ..schema import ONNXSchema, ONNXParameterType, SCHEMAS
-from .node_utils import parse_variadic_param
+from ..schema import ONNXParameter, ONNXSchema, ONNXParameterType, SCHEMAS
+from .node_utils import is_variadic_connector, parse_variadic_param
 
 log = logging.getLogger(__name__)
 
 
-def get_missing_arguments_message(function_name, missing_arguments, argument_type):
-    names = list(map(lambda x: "'" + x + "'", missing_arguments))
-    if len(missing_arguments) == 1:
-        arglist = names[0]
-    else:
-        arglist = ", ".join(names[:-1]) + ", and " + names[-1]
-    return "{function_name} missing {num_missing} required {argument_type}{s}: {arglist}".format(
-        function_name=function_name, num_missing=len(missing_arguments), argument_type=argument_type,
-        s='' if len(missing_arguments) == 1 else 's', arglist=arglist)
+def _missing_message(owner: str, names: typing.Sequence[str], kind: str) -> str:
+    """Worded like Python's own report of missing arguments."""
+    quoted = [f"'{n}'" for n in names]
+    listing = quoted[0] if len(quoted) == 1 else ", ".join(quoted[:-1]) + ", and " + quoted[-1]
+    return f"{owner} missing {len(names)} required {kind}{'' if len(names) == 1 else 's'}: {listing}"
 
 
 def _is_private(connector: str) -> bool:
+    # connectors with a leading underscore belong to one implementation (operands folded in by the
+    # fusion pass); they are not schema parameters
     return connector.startswith("_")
+
+
+class _Binding(typing.NamedTuple):
+    """One edge of a node matched against its schema."""
+    edge: MultiConnectorEdge
+    is_input: bool
+    connector: str
+    parameter: typing.Optional[ONNXParameter]   # None: the schema has no parameter of that name
+    index: typing.Optional[int]                 # position inside a variadic parameter
+    position: typing.Tuple[int, int]            # sort key: (place in the schema, variadic index)
 
 
 class ExpansionRefused(NotImplementedError):
@@ -56,137 +63,103 @@ class ONNXOp(LibraryNode):
                 return call_onnx_op(cls, **kwargs)
         return super().__new__(cls)
 
-    # ---- edges in schema order (onnx_op.py:107-189) ----------------------------------
-    def iter_outputs_in_onnx_order(self, state: SDFGState) -> typing.List[MultiConnectorEdge]:
-        return self._iter_params_in_onnx_order(state, inputs=False)
+    # ---- edges matched against the schema ---------------------------------------------------
+    def _bindings(self, state: SDFGState, inputs: bool) -> typing.List[_Binding]:
+        """The node's (public) edges on one side, each resolved to its schema parameter, in schema order."""
+        parameters = self.schema.inputs if inputs else self.schema.outputs
+        place = {p.name: i for i, p in enumerate(parameters)}
+        found = []
+        for edge in (state.in_edges(self) if inputs else state.out_edges(self)):
+            connector = edge.dst_conn if inputs else edge.src_conn
+            if connector is None:
+                raise ValueError("Edges to ONNX Ops must not have connector None")
+            if _is_private(connector):
+                continue
+            base, index = parse_variadic_param(connector) if is_variadic_connector(connector) else (connector, None)
+            parameter = parameters[place[base]] if base in place else None
+            found.append(_Binding(edge, inputs, connector, parameter, index,
+                                  (place.get(base, len(parameters)), index or 0)))
+        found.sort(key=lambda b: b.position)
+        return found
 
     def iter_inputs_in_onnx_order(self, state: SDFGState) -> typing.List[MultiConnectorEdge]:
-        return self._iter_params_in_onnx_order(state, inputs=True)
+        """Input edges ordered as the schema orders its parameters (``onnx_op.py:107-125``)."""
+        return [b.edge for b in self._bindings(state, True) if b.parameter is not None]
 
-    def _iter_params_in_onnx_order(self, state, inputs=False):
-        parameters = list(self.schema.inputs if inputs else self.schema.outputs)
-        if len(parameters) == 0:
-            return []
-        if parameters[-1].param_type == ONNXParameterType.Variadic:
-            name = parameters[-1].name
-            names = itertools.chain([p.name for p in parameters[:-1]],
-                                    (name + "__" + str(i) for i in itertools.count()))
-        else:
-            names = [p.name for p in parameters]
-        edges = state.in_edges(self) if inputs else state.out_edges(self)
-        conn_to_edge = {(e.dst_conn if inputs else e.src_conn): e for e in edges}
-        out = []
-        for n in itertools.islice(names, len(parameters) + len(edges)):
-            if n in conn_to_edge:
-                out.append(conn_to_edge[n])
-        return out
+    def iter_outputs_in_onnx_order(self, state: SDFGState) -> typing.List[MultiConnectorEdge]:
+        return [b.edge for b in self._bindings(state, False) if b.parameter is not None]
 
     def iter_edges(self, state: SDFGState):
-        """(edge, is_input) pairs ordered as the schema orders its parameters."""
-        def get_idx(parameters, name):
-            number = 0
-            if '__' in name:
-                name, number = parse_variadic_param(name)
-            matched = [i for i, param in enumerate(parameters) if param.name == name]
-            if len(matched) != 1:
-                raise ValueError("Found {} connectors with name '{}', expected to find exactly one".format(
-                    len(matched), name))
-            return matched[0] + number
+        """(edge, is_input) pairs, inputs first, each side in schema order (``onnx_op.py:127-189``)."""
+        for inputs in (True, False):
+            for b in self._bindings(state, inputs):
+                if b.parameter is None:
+                    raise ValueError(f"Found 0 connectors with name '{b.connector}', expected to find exactly one")
+                yield b.edge, inputs
 
-        # connectors with a leading underscore are private to an implementation (operands
-        # folded in by the fusion pass); they are not schema parameters
-        sorted_in = sorted((e for e in state.in_edges(self) if not _is_private(e.dst_conn)),
-                           key=lambda e: get_idx(self.schema.inputs, e.dst_conn))
-        sorted_out = sorted((e for e in state.out_edges(self) if not _is_private(e.src_conn)),
-                            key=lambda e: get_idx(self.schema.outputs, e.src_conn))
-        return itertools.chain(zip(sorted_in, itertools.repeat(True)), zip(sorted_out, itertools.repeat(False)))
-
-    # ---- validation (onnx_op.py:197-415) ------------------------------------------------
+    # ---- validation: the contract of ``onnx_op.py:197-415`` ----------------------------------
+    # every edge names a parameter of the schema and a connector of the node; every required parameter is
+    # connected; the indices of a variadic parameter are 0..n-1, each once; all parameters that share a type
+    # string carry one dtype, and it is one the schema allows; required attributes are set.
     def validate(self, sdfg: SDFG, state: SDFGState):
-        in_edges = state.in_edges(self)
-        out_edges = state.out_edges(self)
+        sides = [(True, self._bindings(state, True)), (False, self._bindings(state, False))]
+        for checker in (self._check_names, self._check_required, self._check_variadic_numbering):
+            for inputs, bindings in sides:
+                checker(inputs, bindings)
+        self._check_dtypes(sdfg, [b for _, bindings in sides for b in bindings])
+        unset = [name for name, attr in self.schema.attributes.items() if attr.required and getattr(self, name) is None]
+        if unset:
+            raise ValueError(f"Expected value for required attribute '{unset[0]}', got None")
 
-        all_connectors = {e.dst_conn for e in in_edges}.union(e.src_conn for e in out_edges)
-        if None in all_connectors:
-            raise ValueError("Edges to ONNX Ops must not have connector None")
-        in_edges = [e for e in in_edges if not _is_private(e.dst_conn)]
-        out_edges = [e for e in out_edges if not _is_private(e.src_conn)]
+    def _check_names(self, inputs: bool, bindings: typing.List[_Binding]):
+        kind = "input" if inputs else "output"
+        declared = self.in_connectors if inputs else self.out_connectors
+        for b in bindings:
+            if b.parameter is None:
+                if b.index is None:
+                    raise TypeError(f"Got an unexpected argument '{b.connector}'")
+                raise ValueError(f"Got an unexpected variadic argument '{b.connector}'")
+            if (b.index is not None) != (b.parameter.param_type == ONNXParameterType.Variadic):
+                if b.index is not None:
+                    raise ValueError(f"Got variadic argument '{b.connector}' for non-variadic parameter "
+                                     f"'{b.parameter.name}'. Ensure that non-variadic args do not contain '__'")
+                raise ValueError(f"Got an unexpected variadic argument '{b.connector}': variadic parameter "
+                                 f"'{b.parameter.name}' is connected as '{b.parameter.name}__<index>'")
+            if b.connector not in declared:
+                raise ValueError(f"Memlet {b.edge.data} leading to nonexistent {kind} connector '{b.connector}'")
 
-        known_inputs = {inp.name for inp in self.schema.inputs}
-        known_outputs = {outp.name for outp in self.schema.outputs}
-        passed_inputs = {e.dst_conn for e in in_edges if '__' not in e.dst_conn}
-        passed_outputs = {e.src_conn for e in out_edges if '__' not in e.src_conn}
+    def _check_required(self, inputs: bool, bindings: typing.List[_Binding]):
+        connected = {b.parameter.name for b in bindings}
+        missing = sorted(p.name for p in (self.schema.inputs if inputs else self.schema.outputs)
+                         if p.param_type == ONNXParameterType.Single and p.name not in connected)
+        if missing:
+            raise ValueError(_missing_message(self.schema.name, missing, "input" if inputs else "output"))
 
-        unknown_inputs = passed_inputs.difference(known_inputs)
-        if len(unknown_inputs) > 0:
-            raise TypeError("Got an unexpected argument '{}'".format(sorted(unknown_inputs)[0]))
-        unknown_outputs = passed_outputs.difference(known_outputs)
-        if len(unknown_outputs) > 0:
-            raise TypeError("Got an unexpected argument '{}'".format(sorted(unknown_outputs)[0]))
+    @staticmethod
+    def _check_variadic_numbering(inputs: bool, bindings: typing.List[_Binding]):
+        kind = "inputs" if inputs else "outputs"
+        indices = [b.index for b in bindings if b.index is not None]   # at most one variadic parameter per side
+        for number in indices:
+            if indices.count(number) > 1:
+                raise ValueError(f"Got two variadic {kind} with index {number}, expected at most one")
+        for expected in range(len(indices)):
+            if expected not in indices:
+                raise ValueError(f"Since {len(indices)} variadic {kind} were passed, "
+                                 f"expected variadic parameter with number {expected}")
 
-        for edge, is_input in self.iter_edges(state):
-            conn_name = edge.dst_conn if is_input else edge.src_conn
-            if conn_name not in (self.in_connectors if is_input else self.out_connectors):
-                raise ValueError("Memlet {} leading to nonexistent {} connector '{}'".format(
-                    edge.data, "input" if is_input else "output", conn_name))
-
-        required_inputs = {i.name for i in self.schema.inputs if i.param_type == ONNXParameterType.Single}
-        missing_inputs = required_inputs.difference(passed_inputs)
-        if len(missing_inputs) > 0:
-            raise ValueError(get_missing_arguments_message(self.schema.name, sorted(missing_inputs), "input"))
-        required_outputs = {o.name for o in self.schema.outputs if o.param_type == ONNXParameterType.Single}
-        missing_outputs = required_outputs.difference(passed_outputs)
-        if len(missing_outputs) > 0:
-            raise ValueError(get_missing_arguments_message(self.schema.name, sorted(missing_outputs), "output"))
-
-        for is_input, edges, params in ((True, in_edges, self.schema.inputs), (False, out_edges, self.schema.outputs)):
-            variadic = {p.name for p in params if p.param_type == ONNXParameterType.Variadic}
-            passed = {(e.dst_conn if is_input else e.src_conn) for e in edges}
-            passed = {c for c in passed if '__' in c}
-            seen = set()
-            for param in passed:
-                name, number = parse_variadic_param(param)
-                if name not in variadic:
-                    raise ValueError("Got an unexpected variadic argument '{}'".format(param))
-                if number in seen:
-                    raise ValueError("Got two variadic {} with index {}, expected at most one".format(
-                        "inputs" if is_input else "outputs", number))
-                seen.add(number)
-            for i in range(len(seen)):
-                if i not in seen:
-                    raise ValueError("Since {} variadic {} were passed, expected variadic parameter with number {}"
-                                     .format(len(seen), "inputs" if is_input else "outputs", i))
-
-        # type constraints must solve
-        assigned_params = {}
-        for edge, is_input in self.iter_edges(state):
-            conn_name = edge.dst_conn if is_input else edge.src_conn
-            parsed_name = parse_variadic_param(conn_name)[0] if '__' in conn_name else conn_name
-            matching = [p for p in (self.schema.inputs if is_input else self.schema.outputs) if p.name == parsed_name]
-            if len(matching) != 1:
-                raise ValueError("Expected to find one {} parameter in schema with name '{}', but found {}".format(
-                    "input" if is_input else "output", parsed_name, len(matching)))
-            matched = matching[0]
-            if '__' in conn_name and matched.param_type != ONNXParameterType.Variadic:
-                raise ValueError("Got variadic argument '{}' for non-variadic parameter '{}'."
-                                 " Ensure that non-variadic args do not contain '__'".format(conn_name, matched.name))
-            edge_dtype = sdfg.arrays[edge.data.data].dtype
-            if matched.type_str in assigned_params and assigned_params[matched.type_str] != edge_dtype:
-                raise ValueError("Could not solve type constraints;"
-                                 " excepted type '{expected}' for {param_type} '{conn_name}', got type '{actual}'".format(
-                                     expected=assigned_params[matched.type_str],
-                                     param_type="input" if is_input else "output",
-                                     conn_name=matched.name, actual=edge_dtype))
-            cons = self.schema.type_constraints[matched.type_str]
-            if edge_dtype not in cons.types:
-                raise ValueError("Expected type in '{possible}' for {param_type} '{conn_name}', got type '{actual}'".format(
-                    possible=cons.types, param_type="input" if is_input else "output",
-                    conn_name=matched.name, actual=edge_dtype))
-            assigned_params[matched.type_str] = edge_dtype
-
-        for name, attr in self.schema.attributes.items():
-            if attr.required and getattr(self, name) is None:
-                raise ValueError("Expected value for required attribute '{}', got None".format(name))
+    def _check_dtypes(self, sdfg: SDFG, bindings: typing.List[_Binding]):
+        solved = {}   # type string -> dtype
+        for b in bindings:
+            kind = "input" if b.is_input else "output"
+            dtype = sdfg.arrays[b.edge.data.data].dtype
+            type_str = b.parameter.type_str
+            allowed = self.schema.type_constraints[type_str].types
+            if dtype != solved.get(type_str, dtype):
+                raise ValueError(f"Could not solve type constraints; excepted type '{solved[type_str]}' for {kind} "
+                                 f"'{b.parameter.name}', got type '{dtype}'")
+            if dtype not in allowed:
+                raise ValueError(f"Expected type in '{allowed}' for {kind} '{b.parameter.name}', got type '{dtype}'")
+            solved[type_str] = dtype
 
 
 # ------------------------------------------------------------------------------------
@@ -280,7 +253,7 @@ def _make_class(dace_schema: ONNXSchema):
             raise TypeError("__init__() takes 1 positional arguments but {} were given".format(1 + len(args)))
         missing_arguments = required_attrs.difference(op_attributes)
         if len(missing_arguments) > 0:
-            raise TypeError(get_missing_arguments_message("__init__()", sorted(missing_arguments),
+            raise TypeError(_missing_message("__init__()", sorted(missing_arguments),
                                                           "keyword-only argument"))
         unknown_attrs = set(op_attributes).difference(dace_schema.attributes)
         if len(unknown_attrs) > 0:

@@ -36,20 +36,16 @@ def empty_sdfg_for_node(sdfg: SDFG, state: SDFGState, node, add_access_nodes=Tru
     """
     nsdfg = SDFG(node.label + "_expansion")
     nstate = nsdfg.add_state()
-    input_nodes, output_nodes = {}, {}
+    access = {True: {}, False: {}}   # is_input -> connector -> access node
     for edge, is_input in node.iter_edges(state):
-        if is_input:
-            conn_name = edge.dst_conn
-            nsdfg.add_datadesc(conn_name, copy.deepcopy(in_desc_with_name(node, state, sdfg, conn_name)))
-            if add_access_nodes:
-                input_nodes[conn_name] = nstate.add_read(conn_name)
-        else:
-            conn_name = edge.src_conn
-            nsdfg.add_datadesc(conn_name, copy.deepcopy(out_desc_with_name(node, state, sdfg, conn_name)))
-            if add_access_nodes:
-                output_nodes[conn_name] = nstate.add_write(conn_name)
-        nsdfg.arrays[conn_name].transient = False
-    return nsdfg, nstate, input_nodes, output_nodes
+        connector = edge.dst_conn if is_input else edge.src_conn
+        outer = (in_desc_with_name if is_input else out_desc_with_name)(node, state, sdfg, connector)
+        inner = copy.deepcopy(outer)
+        inner.transient = False
+        nsdfg.add_datadesc(connector, inner)
+        if add_access_nodes:
+            access[is_input][connector] = (nstate.add_read if is_input else nstate.add_write)(connector)
+    return nsdfg, nstate, access[True], access[False]
 
 
 def kernel_call_for_node(node, state: SDFGState, function: str, args) -> dace.KernelCall:

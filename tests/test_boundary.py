@@ -152,6 +152,63 @@ def test_validate_errors():
         sdfg.expand_library_nodes()
 
 
+def test_validate_variadic_parameters_and_connectors():
+    """The rest of the validation contract (onnx_op.py:197-415): variadic connectors are numbered 0..n-1 without
+    gaps, `__` belongs to variadic parameters only, every edge ends on a declared connector, required attributes
+    are set, and the edges come back in schema order whatever order they were added in."""
+    f32 = dace.float32
+    ok = {"data_0__1": ([4], f32), "data_0__0": ([4], f32), "data_0__2": ([4], f32)}
+    node = donnx.ONNXSum("s")
+    sdfg, st = _one_node_sdfg(node, ok, {"sum": ([4], f32)})
+    node.validate(sdfg, st)
+    assert [e.dst_conn for e in node.iter_inputs_in_onnx_order(st)] == ["data_0__0", "data_0__1", "data_0__2"]
+    assert [(e.dst_conn if i else e.src_conn) for e, i in node.iter_edges(st)] == ["data_0__0", "data_0__1", "data_0__2", "sum"]
+    node = donnx.ONNXSum("s")
+    sdfg, st = _one_node_sdfg(node, {"data_0__0": ([4], f32), "data_0__2": ([4], f32)}, {"sum": ([4], f32)})
+    with pytest.raises(ValueError, match="expected variadic parameter with number 1"):
+        node.validate(sdfg, st)
+    node = donnx.ONNXSum("s")
+    sdfg, st = _one_node_sdfg(node, {"data_0__0": ([4], f32), "other__1": ([4], f32)}, {"sum": ([4], f32)})
+    with pytest.raises(ValueError, match="unexpected variadic argument 'other__1'"):
+        node.validate(sdfg, st)
+    node = donnx.ONNXSum("s")
+    sdfg, st = _one_node_sdfg(node, {"data_0__00": ([4], f32)}, {"sum": ([4], f32)})
+    with pytest.raises(ValueError, match="leading zeroes"):
+        node.validate(sdfg, st)
+    node = donnx.ONNXRelu("r")
+    sdfg, st = _one_node_sdfg(node, {"X__0": ([4], f32)}, {"Y": ([4], f32)})
+    with pytest.raises(ValueError, match="non-variadic parameter 'X'"):
+        node.validate(sdfg, st)
+    # an edge on a connector the node does not declare
+    node = donnx.ONNXConv("c")
+    sdfg, st = _one_node_sdfg(node, {"X": ([1, 1, 4, 4], f32), "W": ([1, 1, 3, 3], f32), "B": ([1], f32)}, {"Y": ([1, 1, 2, 2], f32)})
+    node.validate(sdfg, st)
+    node.remove_in_connector("B")
+    with pytest.raises(ValueError, match="nonexistent input connector 'B'"):
+        node.validate(sdfg, st)
+    # inputs in schema order although W was connected before X
+    node = donnx.ONNXConv("c")
+    sdfg, st = _one_node_sdfg(node, {"W": ([1, 1, 3, 3], f32), "X": ([1, 1, 4, 4], f32)}, {"Y": ([1, 1, 2, 2], f32)})
+    assert [e.dst_conn for e in node.iter_inputs_in_onnx_order(st)] == ["X", "W"]
+    # missing output, several missing inputs
+    node = donnx.ONNXGemm("g")
+    sdfg, st = _one_node_sdfg(node, {}, {"Y": ([2, 2], f32)})
+    with pytest.raises(ValueError, match="Gemm missing 2 required inputs: 'A', and 'B'"):
+        node.validate(sdfg, st)
+    node = donnx.ONNXRelu("r")
+    sdfg, st = _one_node_sdfg(node, {"X": ([4], f32)}, {})
+    with pytest.raises(ValueError, match="Relu missing 1 required output: 'Y'"):
+        node.validate(sdfg, st)
+    # a required attribute left unset
+    node = donnx.ONNXCast("c", to=1)
+    node.to = None
+    sdfg, st = _one_node_sdfg(node, {"input": ([4], f32)}, {"output": ([4], f32)})
+    with pytest.raises(ValueError, match="required attribute 'to'"):
+        node.validate(sdfg, st)
+    with pytest.raises(TypeError, match="missing 1 required keyword-only argument: 'to'"):
+        donnx.ONNXCast("c")
+
+
 @pytest.mark.parametrize("case", ["matmul_1d", "conv_group", "conv_3d", "mmi_zp_wrong_length", "gelu_tanh", "ln_mean_out",
                                   "softmax_f64", "gemm_beta"])
 def test_refusal_is_an_error_not_a_fallback(case):
