@@ -96,10 +96,14 @@ class ONNXModel:
             model = proto.load(model)
         if storage is not None and "GPU" not in str(storage):
             raise ValueError(f"storage {storage!r}: this runner keeps every array in GPU global memory")
+        default_opset = 12
         for opset in model.opset_import:
-            if opset.domain == "" and opset.version not in (12, 17, 20):
-                log.warning(f"Expected the onnx model to be exported with opset 12, got {opset.version}. "
-                            f"This model may fail to import as a result.")
+            if opset.domain in ("", "ai.onnx"):
+                default_opset = opset.version
+                if opset.version not in (12, 17, 20):
+                    log.warning(f"Expected the onnx model to be exported with opset 12, got {opset.version}. "
+                                f"This model may fail to import as a result.")
+        self.opset_version = default_opset  #: version of the default operator set the model imports
         self.do_auto_optimize = auto_optimize
         self.fuse = fuse
         self.use_hip_graph = use_hip_graph
@@ -156,6 +160,10 @@ class ONNXModel:
             if not has_onnx_node(node.op_type):
                 raise ValueError("Unsupported ONNX operator: '{}'".format(node.op_type))
             op_attributes = {a.name: self._convert_attribute(a) for a in node.attribute}
+            # Softmax / LogSoftmax without an axis attribute: the node classes carry the opset-11 default (1);
+            # from opset 13 on the operator's default is the last axis
+            if node.op_type in ("Softmax", "LogSoftmax") and "axis" not in op_attributes and self.opset_version >= 13:
+                op_attributes["axis"] = -1
             node_name = clean_onnx_name(node.name) if node.name else node.op_type + "_" + str(i)
             op_node = get_onnx_node(node.op_type)(node_name, **op_attributes)
             self.state.add_node(op_node)

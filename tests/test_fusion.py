@@ -377,3 +377,20 @@ def test_tasklet_fusion_programs_become_one_launch():
         calls = _launches(donnx.ONNXModel("tf_" + name, m))
         assert [f for f, _ in calls] == ["mi355x_eltwise_program_f32"], name
         assert calls[0][1][1] == len(inputs) and calls[0][1][8] == len(m.graph.node)     # tensors read, instructions
+
+
+@pytest.mark.parametrize("opset, expected", [(12, (2, 3, 8)), (13, (6, 8, 1)), (17, (6, 8, 1))])
+@pytest.mark.parametrize("op", ["Softmax", "LogSoftmax"])
+def test_softmax_without_axis_attribute_takes_the_default_of_the_models_opset(op, opset, expected):
+    """The operator's default axis is 1 up to opset 12 and the last axis from opset 13 on; the reference only
+    ever sees opset 12 (daceml/pytorch/module.py:248), this importer also accepts 17 and 20."""
+    g = H.make_graph([H.make_node(op, ["x"], ["y"])], "g", [H.make_tensor_value_info("x", 1, [2, 3, 8])],
+                     [H.make_tensor_value_info("y", 1, [2, 3, 8])])
+    calls = _launches(donnx.ONNXModel(f"{op}_{opset}", H.make_model(g, opset_imports=[H.make_opsetid("", opset)])))
+    assert len(calls) == 1 and calls[0][0] == ("mi355x_softmax_f32" if op == "Softmax" else "mi355x_log_softmax_f32")
+    assert tuple(calls[0][1][2:5]) == expected   # outer, axis_len, inner
+    # an explicit attribute wins in every opset
+    g = H.make_graph([H.make_node(op, ["x"], ["y"], axis=0)], "g", [H.make_tensor_value_info("x", 1, [2, 3, 8])],
+                     [H.make_tensor_value_info("y", 1, [2, 3, 8])])
+    calls = _launches(donnx.ONNXModel(f"{op}_{opset}_a0", H.make_model(g, opset_imports=[H.make_opsetid("", opset)])))
+    assert tuple(calls[0][1][2:5]) == (1, 2, 24)

@@ -414,3 +414,123 @@ def test_bert_layer_against_transformers():
         ref = layer(t(x))
         ref = (ref[0] if isinstance(ref, (tuple, list)) else ref).numpy()
     assert rel_err(ref, O.bert_layer(x, w, heads=heads)) < 5e-6
+
+
+# ----------------------------------------------------------------------------- Slice, Cast, Einsum (checker functions of the widening operators)
+def _onnx_slice_indices(dim, start, end, step):
+    """Index list of one axis by the ONNX Slice rules, written out without Python slicing: negative start / end
+    count from the end, then start is clamped to [0, dim] (step > 0) or [0, dim - 1] (step < 0) and end to
+    [0, dim] or [-1, dim - 1]."""
+    assert step != 0
+    if start < 0:
+        start += dim
+    if end < 0:
+        end += dim
+    if step > 0:
+        start = min(max(start, 0), dim)
+        end = min(max(end, 0), dim)
+    else:
+        start = min(max(start, 0), dim - 1)
+        end = min(max(end, -1), dim - 1)
+    out, i = [], start
+    while (i < end) if step > 0 else (i > end):
+        out.append(i)
+        i += step
+    return out
+
+
+def test_slice_against_explicit_index_loops():
+    INT64_MAX, INT64_MIN = 2**63 - 1, -2**63
+    rng = np.random.default_rng(40)
+    data = rng.normal(size=(5, 7, 4)).astype(np.float32)
+    cases = [
+        ([1], [4], None, None), ([0], [INT64_MAX], [0], None), ([2], [INT64_MAX], [1], [1]),
+        ([-3], [INT64_MAX], [1], [1]), ([1, 0], [100, -1], [0, 2], [1, 1]), ([0, 1, 1], [5, 7, 3], [0, 1, 2], [2, 3, 1]),
+        ([6], [0], [1], [-1]), ([6], [INT64_MIN], [1], [-1]), ([-1], [INT64_MIN], [1], [-2]), ([100], [-100], [1], [-3]),
+        ([3], [3], [0], [1]), ([4], [2], [0], [1]), ([-100], [2], [0], [1]), ([1], [3], [-1], [1]), ([3, 5], [0, 1], [-1, -2], [-1, -2]),
+    ]
+    for starts, ends, axes, steps in cases:
+        ax = list(range(len(starts))) if axes is None else [a % data.ndim for a in axes]
+        st = [1] * len(starts) if steps is None else steps
+        picks = [list(range(d)) for d in data.shape]
+        for s, e, a, t in zip(starts, ends, ax, st):
+            picks[a] = _onnx_slice_indices(data.shape[a], s, e, t)
+        expected = np.empty([len(p) for p in picks], np.float32)
+        for i, pi in enumerate(picks[0]):
+            for j, pj in enumerate(picks[1]):
+                for k, pk in enumerate(picks[2]):
+                    expected[i, j, k] = data[pi, pj, pk]
+        got = O.slice_(data, starts, ends, axes, steps)
+        assert got.shape == expected.shape and np.array_equal(got, expected), (starts, ends, axes, steps)
+
+
+def test_cast_truncates_toward_zero_and_to_bool():
+    x = np.array([0.5, -0.5, 1.5, -1.5, 2.9, -2.9, 3.0, -3.0, 0.0, -0.0, 1e-30, 255.9, -128.9, 65536.7], np.float32)
+    toward_zero = [int(v) for v in x.tolist()]   # Python's int() truncates toward zero
+    assert toward_zero[:8] == [0, 0, 1, -1, 2, -2, 3, -3]
+    assert O.cast(x, np.int32).tolist() == toward_zero
+    assert O.cast(x, np.int64).tolist() == toward_zero
+    assert O.cast(x[:12], np.int16).tolist() == toward_zero[:12]
+    assert O.cast(x, np.bool_).tolist() == [v != 0 for v in x.tolist()]
+    i = np.array([-2**24, -1, 0, 1, 2**24, 123456], np.int32)
+    assert O.cast(i, np.float32).tolist() == [float(v) for v in i.tolist()] and O.cast(i, np.float32).dtype == np.float32
+    assert O.cast(np.array([True, False]), np.float32).tolist() == [1.0, 0.0]
+    d = np.array([1.0 + 2.0**-30, 0.1], np.float64)
+    assert O.cast(d, np.float32).tolist() == [1.0, float(np.float32(0.1))]
+
+
+def _einsum_brute(equation, a, b):
+    ins, out = equation.replace(" ", "").split("->")
+    ia, ib = ins.split(",")
+    size = {}
+    for letters, arr in ((ia, a), (ib, b)):
+        for letter, n in zip(letters, arr.shape):
+            assert size.setdefault(letter, n) == n
+    letters = sorted(size)
+    result = np.zeros([size[c] for c in out], np.float64)
+    idx = dict.fromkeys(letters, 0)
+
+    def walk(depth):
+        if depth == len(letters):
+            result[tuple(idx[c] for c in out)] += float(a[tuple(idx[c] for c in ia)]) * float(b[tuple(idx[c] for c in ib)])
+            return
+        for v in range(size[letters[depth]]):
+            idx[letters[depth]] = v
+            walk(depth + 1)
+
+    walk(0)
+    return result
+
+
+def test_einsum_against_brute_force_index_loops():
+    rng = np.random.default_rng(41)
+    shapes = {"i": 3, "j": 4, "k": 2, "b": 2, "h": 3, "d": 4}
+    for eq in ("ik,kj->ij", "bik,kj->bij", "bik,bkj->bij", "bhid,bhjd->bhij", "ik,jk->ij", "ki,kj->ji", "bij,bjk->bki",
+               "i,i->i", "ij,j->i"):
+        ia, ib = eq.split("->")[0].split(",")
+        a = rng.normal(size=[shapes[c] for c in ia]).astype(np.float32)
+        b = rng.normal(size=[shapes[c] for c in ib]).astype(np.float32)
+        got = O.einsum(eq, a, b)
+        want = _einsum_brute(eq, a, b)
+        assert got.shape == want.shape and np.allclose(got, want, rtol=1e-5, atol=1e-6), eq
+    # a transposed operand or a swapped output must not go unnoticed
+    a, b = rng.normal(size=(3, 3)).astype(np.float32), rng.normal(size=(3, 3)).astype(np.float32)
+    assert not np.allclose(O.einsum("ik,kj->ij", a, b), _einsum_brute("ik,jk->ij", a, b))
+    assert not np.allclose(O.einsum("ik,kj->ij", a, b), _einsum_brute("ik,kj->ji", a, b))
+
+
+def test_elementwise_pass_throughs_against_the_math_module():
+    """sub, mul, div, sqrt are one-line numpy calls in the checker; pin them value by value."""
+    import math
+    rng = np.random.default_rng(42)
+    a = rng.normal(size=(3, 5)).astype(np.float32)
+    b = (rng.normal(size=5) + 3).astype(np.float32)
+    for name, fn in (("sub", lambda x, y: x - y), ("mul", lambda x, y: x * y), ("div", lambda x, y: x / y)):
+        got = getattr(O, name)(a, b)
+        for i in range(3):
+            for j in range(5):
+                assert got[i, j] == np.float32(fn(np.float32(a[i, j]), np.float32(b[j]))), name
+    s = O.sqrt(np.abs(a))
+    for i in range(3):
+        for j in range(5):
+            assert abs(float(s[i, j]) - math.sqrt(abs(float(a[i, j])))) <= 1e-7 * max(1.0, float(s[i, j]))
