@@ -8,7 +8,7 @@ Layout (mirrors the part of ``daceml`` that lies on the expansion hot path):
 ``onnx``                        ``ONNXForward`` registry, ``ONNX<Op>`` library nodes, the ``"mi355x"``
                                 implementations and the ``ONNXModel`` runner (``import dace_onnx_amd.onnx as donnx``)
 ``util``                        ``in_desc_with_name`` / ``expand_onnx_nodes`` / ``auto_optimize``
-``testing``                     ``torch_tensors_close`` and the event timer
+``testing``                     ``torch_tensors_close``; ``testing.profiling``: HIP-event timers
 """
 import logging
 import os

@@ -451,7 +451,10 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
         }
     };
     // zero points when there is one value per operand (read once, wave-uniform)
-    const uint32_t za_one = ZP ? (uint32_t)a_zero_point(p, 0) : 0u, zb_one = ZP ? (uint32_t)b_zero_point(p, 0) : 0u;
+    // First zero point of each operand, as the aligned 32-bit word that holds it: loaded behind the first operand transfers (below) and
+    // not looked at before the first tile is finished, so the load (a cold page, typically) never stalls the
+    // pipeline's start. A missing zero point reads a byte of the operand instead (any valid address).
+    uint32_t za_raw = 0u, zb_raw = 0u;
 
     // Y = acc - zb[n] rowsum[m] - za[m] (colsum[n] - K zb[n]); accumulators restart at 0
     auto finish_tile = [&](int ti) __attribute__((always_inline)) {
@@ -463,6 +466,16 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
         const int64_t rows_left = p.M - m0 < BM ? p.M - m0 : BM;
         const __amdgpu_buffer_rsrc_t y_rsrc =
             __builtin_amdgcn_make_buffer_rsrc(p.Y + m0 * p.N + n0, 0, (int)((rows_left * p.N - n0) * 4), 0x00020000);
+        const bool one_each = p.za_stride == 0 && p.zb_stride == 0;   // wave-uniform
+        uint32_t za_one = 0u, zb_one = 0u;
+        if constexpr (ZP) {
+            asm volatile("" : "+v"(za_raw), "+v"(zb_raw));   // keeps the conversion (and the wait for the load) here
+            const int32_t a_bias = AU ? 128 : 0, b_bias = BU ? 128 : 0;
+            const uint32_t za_byte = (za_raw >> (8 * (reinterpret_cast<uintptr_t>(p.za_ptr) & 3))) & 0xffu;
+            const uint32_t zb_byte = (zb_raw >> (8 * (reinterpret_cast<uintptr_t>(p.zb_ptr) & 3))) & 0xffu;
+            za_one = (uint32_t)((p.za_ptr ? (AU ? (int32_t)za_byte : (int32_t)(int8_t)za_byte) : 0) - a_bias);
+            zb_one = (uint32_t)((p.zb_ptr ? (BU ? (int32_t)zb_byte : (int32_t)(int8_t)zb_byte) : 0) - b_bias);
+        }
         const uint32_t row_bytes = (uint32_t)p.N * 4u;
         uint32_t voff[2], zbn[2] = {0u, 0u}, c2[2] = {0u, 0u};
 #pragma unroll
@@ -475,34 +488,51 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
                 c2[t] = (uint32_t)(lds_cols[parity][wn][0][32 * t + lj] + lds_cols[parity][wn][1][32 * t + lj]) - (uint32_t)p.K * zbn[t];
             }
         }
+        // 32-bit integer multiplies run at a quarter of the rate of adds: with one zero point per operand the
+        // correction of an element is two subtractions, y = acc - zb rowsum[m] - za (colsum[n] - K zb)
+        uint32_t d_col[2] = {0u, 0u};
+        if constexpr (ZP) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) d_col[t] = za_one * c2[t];
+        }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            // row sums of the sixteen rows this lane's accumulator registers hold: rows 32 i + 8 q + 4 lg + e
-            i32x4 rs4[4] = {};
             int32_t za_lane = 0;   // zero point of row wm0 + 32 i + lj when there is one per row
             if constexpr (ZP) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    rs4[q] = *reinterpret_cast<const i32x4*>(&lds_rows[parity][wm][0][32 * i + 8 * q + 4 * lg]) +
-                             *reinterpret_cast<const i32x4*>(&lds_rows[parity][wm][1][32 * i + 8 * q + 4 * lg]);
                 if (p.za_stride != 0) {
                     const int64_t m = m0 + wm0 + 32 * i + lj;
                     za_lane = a_zero_point(p, m < p.M ? m : p.M - 1);
                 }
             }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                uint32_t rs = 0, zam = 0;
-                if constexpr (ZP) {
-                    rs = (uint32_t)rs4[r / 4][r % 4];
-                    zam = p.za_stride == 0 ? za_one : (uint32_t)__shfl(za_lane, 8 * (r / 4) + 4 * lg + (r % 4), WAVE);
-                }
-                const uint32_t roff = (uint32_t)(32 * i + 8 * (r / 4) + (r % 4)) * row_bytes;
+            for (int q = 0; q < 4; ++q) {
+                // row sums of the four rows 32 i + 8 q + 4 lg + e that registers 4 q + e hold
+                i32x4 rs4 = {};
+                if constexpr (ZP)
+                    rs4 = *reinterpret_cast<const i32x4*>(&lds_rows[parity][wm][0][32 * i + 8 * q + 4 * lg]) +
+                          *reinterpret_cast<const i32x4*>(&lds_rows[parity][wm][1][32 * i + 8 * q + 4 * lg]);
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const uint32_t y = (uint32_t)acc[i][t][r] - zbn[t] * rs - zam * c2[t];
-                    __builtin_amdgcn_raw_buffer_store_b32((int32_t)y, y_rsrc, (int)(voff[t] + roff), 0, 0);
-                    acc[i][t][r] = 0;
+                for (int e = 0; e < 4; ++e) {
+                    const int r = 4 * q + e;
+                    const uint32_t roff = (uint32_t)(32 * i + 8 * q + e) * row_bytes;
+                    uint32_t y[2] = {(uint32_t)acc[i][0][r], (uint32_t)acc[i][1][r]};
+                    if constexpr (ZP) {
+                        const uint32_t rs = (uint32_t)rs4[e];
+                        if (one_each) {
+                            const uint32_t e_row = zb_one * rs;
+#pragma unroll
+                            for (int t = 0; t < 2; ++t) y[t] = y[t] - e_row - d_col[t];
+                        } else {
+                            const uint32_t zam = p.za_stride == 0 ? za_one : (uint32_t)__shfl(za_lane, 8 * q + 4 * lg + e, WAVE);
+#pragma unroll
+                            for (int t = 0; t < 2; ++t) y[t] = y[t] - zbn[t] * rs - zam * c2[t];
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        __builtin_amdgcn_raw_buffer_store_b32((int32_t)y[t], y_rsrc, (int)(voff[t] + roff), 0, 0);
+                        acc[i][t][r] = 0;
+                    }
                 }
             }
         }
@@ -512,7 +542,14 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     // operand set 0 holds (stage s, first 32 k). A stage is overwritten two steps after it was read.
     issue_loads(0);
     if (total_steps > 1) issue_loads(1);
-    MI355X_WAIT_VMCNT(0);
+    if constexpr (ZP) {
+        // (the aligned word that holds the byte: no conversion instruction, hence no wait, at this point)
+        za_raw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.za_ptr ? p.za_ptr : p.A) & ~(uintptr_t)3);
+        zb_raw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.zb_ptr ? p.zb_ptr : p.B) & ~(uintptr_t)3);
+        MI355X_WAIT_VMCNT(2);   // operations complete in order: the transfers have landed, these two loads may not have
+    } else {
+        MI355X_WAIT_VMCNT(0);
+    }
     __syncthreads();
     read_frags(0, 0, 0);
 
