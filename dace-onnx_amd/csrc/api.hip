@@ -1,7 +1,10 @@
 // Library identity, per-thread error channel and device query.
 #include "common.h"
 
+#include <stdlib.h>
 #include <string.h>
+#include <atomic>
+#include <mutex>
 
 namespace mi355x {
 
@@ -22,9 +25,69 @@ int check_launch(const char* kernel_name) {
     return MI355X_OK;
 }
 
+// ---- launch parameters that do not change from call to call -------------------------------------
+// The MI355X_* variables select kernel variants (used by the tests that run every tile shape) and the CU
+// count sizes persistent grids. Both are looked up once: the environment on first use (again after
+// mi355x_reload_tuning()), the CU count once per device.
+static Tuning g_tuning;
+static std::atomic<bool> g_tuning_valid{false};
+static std::mutex g_tuning_mutex;
+
+static int env_int(const char* name, int fallback) {
+    const char* v = getenv(name);
+    return v && *v ? atoi(v) : fallback;
+}
+
+static void parse_tuning(Tuning& t) {
+    const char* c = getenv("MI355X_GEMM_CONFIG");
+    t.gemm_config = c && c[0] >= '0' && c[0] <= '9' ? c[0] - '0' : -1;
+    t.gemm_nt_bn = env_int("MI355X_GEMM_NT_BN", 0);
+    t.gemm_nt_bk = env_int("MI355X_GEMM_NT_BK", 0);
+    t.gemm_group_m = env_int("MI355X_GEMM_GROUP_M", 0);
+    c = getenv("MI355X_CONV_CONFIG");
+    t.conv_config = c && c[0] >= '0' && c[0] <= '9' ? c[0] - '0' : -1;
+    t.conv_gather_bn = env_int("MI355X_CONV_GATHER_BN", 0);
+    t.mmi_generic = getenv("MI355X_MMI_GENERIC") != nullptr;
+    t.mmi_wgs_per_cu = env_int("MI355X_MMI_WGS_PER_CU", 0);
+}
+
+const Tuning& tuning() {
+    if (!g_tuning_valid.load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_tuning_mutex);
+        if (!g_tuning_valid.load(std::memory_order_relaxed)) {
+            parse_tuning(g_tuning);
+            g_tuning_valid.store(true, std::memory_order_release);
+        }
+    }
+    return g_tuning;
+}
+
+int device_cus() {
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<int> cached[MAX_DEVICES];   // 0: not asked yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (dev < 0 || dev >= MAX_DEVICES) return mi355x_device_cu_count();
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        cus = mi355x_device_cu_count();
+        cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
 }  // namespace mi355x
 
 extern "C" {
+
+void mi355x_reload_tuning(void) {
+    std::lock_guard<std::mutex> lock(mi355x::g_tuning_mutex);
+    mi355x::parse_tuning(mi355x::g_tuning);
+    mi355x::g_tuning_valid.store(true, std::memory_order_release);
+}
 
 int mi355x_version(void) { return MI355X_ONNX_VERSION; }
 

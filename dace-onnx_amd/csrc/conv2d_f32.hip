@@ -469,8 +469,8 @@ static const ConvTile kConvTiles[] = {{64, 128}, {64, 64}, {32, 64}, {16, 64}, {
 constexpr int kNumConvTiles = sizeof(kConvTiles) / sizeof(kConvTiles[0]);
 
 static int choose_conv_tile(int64_t M, int64_t P, int cus) {
-    const char* force = getenv("MI355X_CONV_CONFIG");
-    if (force && force[0] >= '0' && force[0] < '0' + kNumConvTiles) return force[0] - '0';
+    const int force = tuning().conv_config;
+    if (force >= 0 && force < kNumConvTiles) return force;
     double best = 1e300;
     int best_cfg = 1;
     for (int c = 0; c < kNumConvTiles; ++c) {
@@ -539,13 +539,13 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
     p.vec_w = (K % 4 == 0) && al16(W);
     p.vec_y = ((OH * OW) % 4 == 0) && al16(Y) && (!(epilogue & MI355X_EPI_RESIDUAL) || al16(residual));
 
-    int cus = mi355x_device_cu_count();
+    const int cus = device_cus();
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "conv2d: no usable HIP device");
     hipStream_t st = static_cast<hipStream_t>(stream);
     p.group_m = 1;
     // K a multiple of the 32-k tile and 16-byte aligned W rows: the gather kernel
     if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && C * H * Wd < ((int64_t)1 << 27) &&
-        N * C * H * Wd < ((int64_t)1 << 29) && al16(W) && !getenv("MI355X_CONV_CONFIG")) {
+        N * C * H * Wd < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
         p.x_bytes = (int)(N * C * H * Wd * 4);
         // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
         // at the same rate, so the choice is the number of rounds times the tile width; ties go
@@ -554,8 +554,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
             const int64_t tiles = ceil_div(M, (int64_t)CG_BM) * ceil_div(P, (int64_t)bn);
             return ceil_div(tiles, (int64_t)cus * wgs_per_cu) * bn * wgs_per_cu;
         };
-        const bool wide = getenv("MI355X_CONV_GATHER_BN") ? atoi(getenv("MI355X_CONV_GATHER_BN")) == 128
-                                                          : cost(128, 1) < cost(64, 2);
+        const bool wide = tuning().conv_gather_bn ? tuning().conv_gather_bn == 128 : cost(128, 1) < cost(64, 2);
         const int bn = wide ? 128 : 64;
         p.tiles_m = ceil_div(M, (int64_t)CG_BM);
         p.tiles_p = ceil_div(P, (int64_t)bn);

@@ -179,7 +179,7 @@ extern "C" int mi355x_eltwise_program_f32(const float* const* tensors, int n_ten
     }
     const int64_t count = vec ? n / 4 : n;
     int64_t blocks = ceil_div(count, (int64_t)256);
-    const int64_t max_blocks = (int64_t)mi355x_device_cu_count() * 16;
+    const int64_t max_blocks = (int64_t)device_cus() * 16;
     if (max_blocks > 0 && blocks > max_blocks) blocks = max_blocks;
     p.col_step = (uint32_t)((blocks * 256 * (vec ? 4 : 1)) % last_dim);
     hipStream_t st = static_cast<hipStream_t>(stream);

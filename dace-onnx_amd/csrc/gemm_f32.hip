@@ -173,8 +173,8 @@ static void launch_config(int cfg, const GemmArgs& p, bool a_kc, bool b_kc, bool
 // Cost model: time ~ rounds of workgroups over the CUs x work per tile,
 // inflated for small tiles (more LDS/L2 traffic per FLOP) and padding waste.
 static int choose_config(int64_t batch, int64_t M, int64_t N, int64_t K, int cus) {
-    const char* force = getenv("MI355X_GEMM_CONFIG");
-    if (force && force[0] >= '0' && force[0] < '0' + kNumConfigs) return force[0] - '0';
+    const int force = tuning().gemm_config;
+    if (force >= 0 && force < kNumConfigs) return force;
     double best = 1e300;
     int best_cfg = 1;
     for (int c = 0; c < kNumConfigs; ++c) {
@@ -236,11 +236,11 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     if (epilogue & MI355X_EPI_RESIDUAL)
         vec = vec && al16(residual) && m4(p.r_sm) && m4(p.r_sb0) && m4(p.r_sb1);
 
-    int cus = mi355x_device_cu_count();
+    const int cus = device_cus();
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "gemm: no usable HIP device");
     // both operands contiguous along k (activations x pre-transposed weights, Q K^T):
     // the dedicated kernel reads every MFMA fragment with 16-byte accesses
-    if (a_kc && b_kc && vec && !getenv("MI355X_GEMM_CONFIG") && launch_gemm_f32_nt(p, cus, static_cast<hipStream_t>(stream)))
+    if (a_kc && b_kc && vec && tuning().gemm_config < 0 && launch_gemm_f32_nt(p, cus, static_cast<hipStream_t>(stream)))
         return check_launch("gemm_f32_nt_kernel");
     const int cfg = choose_config(batch, M, N, K, cus);
     const TileConfig& tc = kConfigs[cfg];

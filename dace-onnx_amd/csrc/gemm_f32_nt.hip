@@ -268,11 +268,12 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     const Cand cands[] = {{64, 48, 1.0}, {64, 64, 1.0}, {128, 96, 0.8}, {64, 144, 0.9}};
     int best = 0;
     double best_cost = 1e300;
-    const char* force = getenv("MI355X_GEMM_NT_BN");
+    const Tuning& tune = tuning();
+    const int force = tune.gemm_nt_bn;
     for (int c = 0; c < 4; ++c) {
         const int64_t nwg = p.batch * ceil_div(p.M, cands[c].bm) * ceil_div(p.N, cands[c].bn);
         const double cost = (double)ceil_div(nwg, (int64_t)cus) * cands[c].bm * cands[c].bn * cands[c].weight;
-        if (force ? atoi(force) == cands[c].bn : cost < best_cost) { best = c; best_cost = cost; if (force) break; }
+        if (force ? force == cands[c].bn : cost < best_cost) { best = c; best_cost = cost; if (force) break; }
     }
     p.tiles_m = ceil_div(p.M, cands[best].bm);
     p.tiles_n = ceil_div(p.N, cands[best].bn);
@@ -281,14 +282,13 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     // one workgroup per CU at a time: an XCD holds cus / 8 tiles
     const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD);
     p.group_m = choose_group_m(p.tiles_m, per_xcd < cus / NUM_XCD ? per_xcd : cus / NUM_XCD, cands[best].bm, cands[best].bn);
-    if (const char* g = getenv("MI355X_GEMM_GROUP_M")) p.group_m = atoi(g) > 0 ? atoi(g) : 1;
+    if (tune.gemm_group_m > 0) p.group_m = tune.gemm_group_m;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
     // The smallest variant walks K in 64-k tiles with a three-deep ring where K allows: half the barriers per FLOP
     // and the same bytes in flight as six 32-k tiles (1024 x 768 x 768: 14.0 us against 14.7 us, 1024 x 768 x 3072:
     // 41.9 us against 44.8 us with 32-k tiles and 43.9 us with six 64-k tiles in flight; the wider
     // variants lose 1-2 % with 64-k tiles)
-    const char* fbk = getenv("MI355X_GEMM_NT_BK");
-    const bool bk64 = p.K % 64 == 0 && (fbk ? atoi(fbk) == 64 : true);
+    const bool bk64 = p.K % 64 == 0 && (tune.gemm_nt_bk ? tune.gemm_nt_bk == 64 : true);
     if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64, 3>), grid, block, 0, stream, p);
     else if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024

@@ -16,7 +16,6 @@
 #include "gemm_tile.h"
 
 #include <stdlib.h>
-#include <mutex>
 #include <type_traits>
 
 namespace mi355x {
@@ -585,23 +584,6 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     if (pending) finish_tile(tile_i - 1);
 }
 
-// Launch parameters that do not change while the process runs: read once.
-struct MMITuning {
-    int cus = 0;
-    bool force_generic = false;
-    int wgs_per_cu = 3;
-};
-static const MMITuning& mmi_tuning() {
-    static MMITuning t;
-    static std::once_flag once;
-    std::call_once(once, [] {
-        t.cus = mi355x_device_cu_count();
-        t.force_generic = getenv("MI355X_MMI_GENERIC") != nullptr;
-        if (const char* g = getenv("MI355X_MMI_WGS_PER_CU")) t.wgs_per_cu = atoi(g) > 0 ? atoi(g) : 3;
-    });
-    return t;
-}
-
 template <bool ZP>
 static void launch_stream(const MMIArgs& p, int64_t grid, hipStream_t st) {
     const dim3 g((unsigned)grid), b(256);
@@ -642,13 +624,14 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
     auto al = [](const void* q, int a) { return (reinterpret_cast<uintptr_t>(q) & (a - 1)) == 0; };
     hipStream_t st = static_cast<hipStream_t>(stream);
     p.group_m = 1;
-    const MMITuning& tune = mmi_tuning();
+    const Tuning& tune = tuning();
+    const int cus = device_cus();
     // 16-byte transfers of A rows and B rows; a tile's 128 rows of Y are addressed with 31-bit byte offsets
     if (K > 0 && K % MMF_BK == 0 && N % 16 == 0 && al(A, 16) && al(B, 16) && al(Y, 4) && N < ((int64_t)1 << 21) &&
-        !tune.force_generic) {
-        if (tune.cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "matmul_integer: no usable HIP device");
+        !tune.mmi_generic) {
+        if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "matmul_integer: no usable HIP device");
         // persistent grid: three workgroups per CU (a multiple of the XCD count), fewer if there are fewer tiles
-        int64_t grid = (int64_t)tune.wgs_per_cu * (tune.cus / NUM_XCD) * NUM_XCD;
+        int64_t grid = (int64_t)(tune.mmi_wgs_per_cu > 0 ? tune.mmi_wgs_per_cu : 3) * (cus / NUM_XCD) * NUM_XCD;
         if (grid > p.nwg || grid <= 0) grid = p.nwg;
         const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = ceil_div(grid, (int64_t)NUM_XCD);
         p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, MMF_BM, MMF_BN);

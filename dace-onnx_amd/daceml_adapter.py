@@ -113,6 +113,11 @@ def register(ops: typing.Optional[typing.Iterable[str]] = None) -> typing.List[s
 
             @staticmethod
             def forward_can_be_applied(node, state, sdfg):
+                # the kernels take device pointers: every array the node touches has to live in GPU memory
+                touched = [e.data.data for e in list(state.in_edges(node)) + list(state.out_edges(node))
+                           if e.data is not None and e.data.data is not None]
+                if any(sdfg.arrays[name].storage != dace.StorageType.GPU_Global for name in touched):
+                    return False
                 return isinstance(mirror_expansion(node, state, sdfg), light.KernelCall)
 
             @staticmethod

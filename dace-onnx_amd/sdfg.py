@@ -791,6 +791,52 @@ class CompiledSDFG:
     def num_launches(self):
         return sum(1 for item in self._plan if item[0] == "call")
 
+    # -- the same launch sequence as C++ -----------------------------------------------
+    def program_source(self, name: typing.Optional[str] = None) -> typing.Tuple[str, typing.List[str]]:
+        """The launch sequence as a C++ translation unit, the code DaCe would emit around the tasklets of
+        :meth:`KernelCall.as_cpp` (each tasklet a block with ``dace.pointer`` typed connectors ``_<name>``
+        and the stream as ``__dace_current_stream``: ``cudnn_implementations.py:324-334``,
+        ``environments/cudnn.py:44``).
+
+        Returns ``(source, arrays)``. The source includes only ``mi355x_onnx.h`` and defines
+        ``extern "C" int __program_<name>(void** __arrays, void* __dace_current_stream)``; ``arrays`` lists, in
+        the order of ``__arrays``, the arrays whose device pointers the caller passes: the SDFG's non-transient
+        arrays by name, then its transients by their flattened key (see :meth:`transient_descriptors`). A
+        Reshape-like alias of a transient is a pointer assignment; one into caller-owned memory would need a
+        copy and is not supported here.
+        """
+        name = name or self.sdfg.name
+        arrays = list(self._external) + [k for k in self._transients if k not in self._external]
+        index = {k: i for i, k in enumerate(arrays)}
+        desc_of = {**{k: self.sdfg.arrays[k] for k in self._external}, **self._transients}
+        lines = ['#include <stdint.h>', '#include <stdio.h>', '#include <stdlib.h>', '#include "mi355x_onnx.h"', '',
+                 f'extern "C" int __program_{name}(void** __arrays, void* __dace_current_stream) {{']
+        for item in self._plan:
+            if item[0] == "alias":
+                _, src_key, dst_key, _ = item
+                if dst_key in self._external:
+                    raise NotImplementedError(f"alias into caller-owned array '{dst_key}' needs a device copy")
+                if dst_key not in index:
+                    index[dst_key] = len(arrays)
+                    arrays.append(dst_key)
+                lines.append(f"    __arrays[{index[dst_key]}] = __arrays[{index[src_key]}];  // {dst_key} is a view of {src_key}")
+                continue
+            _, node, conn_to_key = item
+            lines.append(f"    {{  // {node.label}")
+            for conn, key in conn_to_key.items():
+                ctype = desc_of[key].dtype.ctype if key in desc_of else "float"
+                lines.append(f"        {ctype}* _{conn} = ({ctype}*)__arrays[{index[key]}];")
+                lines.append(f"        (void)_{conn};")
+            lines.extend("        " + ln for ln in node.as_cpp().splitlines())
+            lines.append("    }")
+        lines += ["    return 0;", "}", ""]
+        return "\n".join(lines), arrays
+
+    def transient_descriptors(self):
+        """Flattened key -> descriptor of every transient array (what :meth:`program_source` expects the caller
+        to allocate besides the SDFG's own arguments)."""
+        return dict(self._transients)
+
     def bound_launches(self):
         """[(KernelCall node, zero-argument callable)] for the currently bound buffers:
         each callable re-issues that one launch on torch's current stream (profiling)."""

@@ -271,6 +271,7 @@ def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
     else:
         monkeypatch.setenv("MI355X_GEMM_NT_BN", tile)
     lib = _lib.library()
+    lib.mi355x_reload_tuning()   # the variables are read once; this test changes them between calls
     rng = np.random.default_rng(M * 7 + N * 3 + K + epi)
     a = torch.from_numpy(rng.normal(size=(2, M, K)).astype(np.float32)).cuda()
     w = torch.from_numpy(rng.normal(size=(N, K)).astype(np.float32)).cuda()          # [N, K]: B[k, n] = w[n, k]
@@ -290,6 +291,8 @@ def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
         ref = torch.nn.functional.gelu(ref)
     if epi & 8:
         ref = ref + res.double()
+    monkeypatch.delenv("MI355X_GEMM_NT_BN", raising=False)
+    lib.mi355x_reload_tuning()   # back to the library's own choice for the tests that follow
     assert rel_err(ref.cpu().numpy(), out.cpu().numpy()) < FP32_REL_TOL
 
 
