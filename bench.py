@@ -28,6 +28,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+WARM_MS = 40.0   # untimed repetitions before every measurement, see dace_onnx_amd/testing/profiling.py
 # published MI355X peaks (dense)
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_INT8_MFMA_TOPS = 5000.0
@@ -36,36 +37,6 @@ PEAK_HBM_GBS = 8000.0
 # this script scaled by a copy kernel of known size (profiles/bert_layer_gemm_traffic.txt); counters cannot be
 # read from inside the process, so the figure is carried here and re-measured whenever the GEMM kernels change
 GEMM_TRAFFIC_BYTES_PER_LAYER = 193172205
-
-
-def graph_time_us(launch, reps=50, replays=5):
-    """Average duration of one launch: `reps` back-to-back launches recorded in a
-    HIP graph (no host launch gaps), replayed between two HIP events on the
-    stream the kernels run on."""
-    import torch
-    launch()  # warm-up, loads the code object
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for _ in range(reps):
-            launch()
-    # warm-up replays for ~40 ms: after a stretch of memory-bound kernels the core clock needs tens of
-    # milliseconds of matrix work to come back up (a cold first measurement of the convolution reads 8 % slow)
-    t_end = time.perf_counter() + 0.040
-    while True:
-        g.replay()
-        torch.cuda.synchronize()
-        if time.perf_counter() >= t_end:
-            break
-    best = float("inf")
-    for _ in range(replays):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        best = min(best, e0.elapsed_time(e1) * 1e3 / reps)
-    return best
 
 
 def algorithmic_work(name, args):
@@ -138,6 +109,7 @@ def main():
     import dace_onnx_amd.onnx as donnx
     from dace_onnx_amd import _lib
     from dace_onnx_amd.testing.graphs import bert_encoder_layer_model
+    from dace_onnx_amd.testing.profiling import graph_time_us, warm_up
     from oracle import pure_ops  # checker / CPU baseline only
 
     if not torch.cuda.is_available():
@@ -190,6 +162,9 @@ def main():
         mode, step = ("eager", eager_step) if t_eager < t_graph else ("graph", compiled.replay)
     else:
         timed(step, args.warmup)
+    # besides the --warmup steps: steps for at least 40 ms, the time the core clock needs to come back up after
+    # idling (every per-kernel row below is warmed the same way, so the headline and the rows are comparable)
+    warm_steps = warm_up(step, WARM_MS)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -211,13 +186,14 @@ def main():
 
     # ---- per-kernel durations, HIP events on the launch stream -----------------------------
     kernels = []
-    gemm_flops = gemm_us = gemm_bytes = 0.0
+    gemm_flops = gemm_us = gemm_bytes = layer_us = 0.0
     if not args.no_kernels:
         for node, relaunch in compiled.bound_launches():
             name = node.function
             plain = [a.values if hasattr(a, "values") else a for a in node.args]
             flops, nbytes = algorithmic_work(name, plain)
             us = graph_time_us(relaunch)
+            layer_us += us   # sum of the layer's kernel durations, to hold against ms_per_step
             if name == "mi355x_gemm_f32":
                 gemm_flops += flops
                 gemm_bytes += nbytes
@@ -308,6 +284,8 @@ def main():
         "config": {"workload": "BASELINE.json configs[2]: BERT-base encoder layer, B=8 S=128 H=768 heads=12 FFN=3072, "
                                "ONNX graph of MatMul/Add/Reshape/Transpose/Div/Softmax/LayerNormalization/Gelu",
                    "launches_per_step": compiled.num_launches, "replay": "host_launches" if mode == "eager" else "hip_graph",
+                   "warm_ms": WARM_MS, "warm_steps": warm_steps,
+                   "kernel_us_per_step": round(layer_us, 2) if layer_us else None,
                    "max_rel_err_vs_oracle": err},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "kernels": kernels,
     }

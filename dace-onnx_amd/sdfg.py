@@ -581,8 +581,8 @@ class SDFG:
 class CompiledSDFG:
     """Executable form of an expanded SDFG: a flat list of kernel launches.
 
-    Transients are allocated once, here. ``__call__`` binds the non-transient
-    arrays, enqueues every launch on torch's current HIP stream and returns
+    Transients are allocated once, when the launch list is first bound, and kept. ``__call__`` binds the
+    non-transient arrays, enqueues every launch on torch's current HIP stream and returns
     without synchronising. ``capture_graph`` records the launches into a HIP
     graph; afterwards ``replay`` re-runs them against the same buffers with a
     single launch.
@@ -599,6 +599,7 @@ class CompiledSDFG:
         self._external = [k for k, d in sdfg.arrays.items() if not d.transient]
         self._written = self._find_written(sdfg)
         self._transients = {}   # flattened key -> descriptor
+        self._transient_tensors = {}   # flattened key -> its allocation (made on first use, kept)
         self._plan = []         # ("call", node, connector -> key) | ("alias", src key, dst key, dst descriptor)
         self._bound_key = None
         self._graph = None
@@ -650,26 +651,35 @@ class CompiledSDFG:
 
     # -- binding ---------------------------------------------------------------------
     def _bind(self, env):
-        """Resolve every pointer argument against ``env`` (key -> tensor)."""
+        """Resolve every pointer argument against ``env`` (key -> tensor). Transient tensors are allocated on the
+        first call and kept: binding again (the caller passed other buffers) only resolves pointers anew."""
         import torch
         env = dict(env)
         launches = []
-        copies = []  # (dst_tensor, src_tensor) for aliases that need a real copy
+        # A Reshape-like alias whose result is caller-owned memory: let the producer of its source write there
+        # directly (the source, a transient, becomes a view of the caller's buffer). Walking the aliases backwards
+        # carries this through chains of them. What cannot be redirected (the source is caller-owned too, or
+        # already a view of something else) is copied on the device.
+        redirected = set()
+        for item in reversed(self._plan):
+            if item[0] != "alias":
+                continue
+            _, src_key, dst_key, _ = item
+            if dst_key in env and src_key not in env and src_key in self._transients:
+                env[src_key] = env[dst_key].reshape(self._transients[src_key].shape)
+                redirected.add((src_key, dst_key))
         for item in self._plan:
             if item[0] == "alias":
                 _, src_key, dst_key, dst_desc = item
-                src = env[src_key]
+                if (src_key, dst_key) in redirected:
+                    continue
+                src = self._tensor(env, src_key)
                 if dst_key in env:
-                    # destination is caller-owned memory: a device copy is needed
                     launches.append(("copy", env[dst_key], src))
                 else:
                     env[dst_key] = src.reshape(dst_desc.shape)  # contiguous -> view
                 continue
             _, node, conn_to_key = item
-            for c, k in conn_to_key.items():
-                if k not in env:
-                    d = self._transients[k]
-                    env[k] = torch.empty(d.shape, dtype=d.dtype.as_torch(), device=self.device)
             fn = getattr(self._lib, node.function)
             args, keep, stream_slots = [], [], []
             for i, a in enumerate(node.args):
@@ -677,7 +687,7 @@ class CompiledSDFG:
                     if a.connector is None:
                         args.append(None)
                     else:
-                        t = env[conn_to_key[a.connector]]
+                        t = self._tensor(env, conn_to_key[a.connector])
                         args.append(t.data_ptr() + a.offset * t.element_size())
                 elif isinstance(a, Stream):
                     stream_slots.append(i)
@@ -688,7 +698,7 @@ class CompiledSDFG:
                     args.append(arr)
                 elif isinstance(a, (U32Array, F32Array, PtrArray)):
                     if isinstance(a, PtrArray):
-                        arr = _lib.pointer_array([env[conn_to_key[c]].data_ptr() for c in a.connectors])
+                        arr = _lib.pointer_array([self._tensor(env, conn_to_key[c]).data_ptr() for c in a.connectors])
                     else:
                         arr = (_lib.u32_array if isinstance(a, U32Array) else _lib.f32_array)(a.values)
                     keep.append(arr)
@@ -697,6 +707,17 @@ class CompiledSDFG:
                     args.append(a)
             launches.append(("call", fn, node.function, args, stream_slots, keep, node))
         return env, launches
+
+    def _tensor(self, env, key):
+        """The tensor bound to ``key``; a transient that has none yet gets its allocation, made once per
+        compiled SDFG and reused by every later binding."""
+        if key not in env:
+            import torch
+            if key not in self._transient_tensors:
+                d = self._transients[key]
+                self._transient_tensors[key] = torch.empty(d.shape, dtype=d.dtype.as_torch(), device=self.device)
+            env[key] = self._transient_tensors[key]
+        return env[key]
 
     def _run(self, launches):
         import torch
@@ -773,8 +794,8 @@ class CompiledSDFG:
         import torch
         if self._bound_key is None:
             raise RuntimeError("call the compiled SDFG once before capturing it")
-        if any(item[0] == "copy" for item in self._launch_list):
-            raise RuntimeError("graphs with caller-owned Reshape outputs are not captured")
+        # (a device copy left over from a Reshape into caller-owned memory is issued on the capture stream like
+        # the kernels and becomes a node of the graph)
         g = torch.cuda.CUDAGraph()
         torch.cuda.synchronize()
         with torch.cuda.graph(g):

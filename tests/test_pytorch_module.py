@@ -185,6 +185,28 @@ def test_lenet_hip_graph_replay(sdfg_name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("use_hip_graph", [False, True])
+def test_module_whose_output_is_a_view_eager_and_as_hip_graph(sdfg_name, use_hip_graph):
+    """A network that ends in Flatten: the graph output is a Reshape of the last kernel's result. The producer
+    writes straight into the output buffer (no copy, nothing that a HIP graph could not hold); several calls,
+    each checked, with the caller keeping earlier results alive (so every eager call sees new output buffers)."""
+    torch.manual_seed(12)
+    net = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1), nn.ReLU(), nn.Flatten()).eval()
+    dace_net = DaceModule(copy.deepcopy(net), sdfg_name=sdfg_name, use_hip_graph=use_hip_graph)
+    kept = []
+    for i in range(4):
+        input = torch.rand(2, 3, 6, 6)
+        out = dace_net(input.cuda())
+        kept.append((net(input), out))
+        torch.cuda.synchronize()
+    for i, (want, got) in enumerate(kept):
+        torch_tensors_close(f"output_{i}", want, got.cpu())
+    compiled = dace_net.dace_model.compile_and_init()
+    assert compiled.num_launches == 1 and not any(item[0] == "copy" for item in compiled._launch_list)
+    assert len(compiled._transient_tensors) <= 1   # allocated once, however many times the outputs changed
+
+
+@pytest.mark.gpu
 def test_lenet(sdfg_name):
     # tests/pytorch/test_lenet.py:37-57
     torch.manual_seed(7)
