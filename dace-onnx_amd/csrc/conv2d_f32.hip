@@ -72,6 +72,8 @@ struct ConvArgs {
     int vec_w;      // W tile may use 16-byte loads
     int vec_y;      // Y may use 16-byte stores (OH*OW % 4 == 0, aligned)
     int x_bytes;    // size of X (gather kernel only; below 2^31)
+    // gather kernel: the first full_tiles workgroups take whole tiles, the rest 16-position slices from p_full on
+    int64_t full_tiles, p_full;
 };
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool VEC_W>
@@ -244,23 +246,26 @@ __device__ __forceinline__ void cg_static_for(F&& f) {
     cg_static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
 
-// TN: 16-position MFMA tiles per wave; BN = 16 TN output positions per workgroup (64 or 128).
+// TN: 16-position MFMA tiles per wave; BN = 16 TN output positions per workgroup: 64 or 128, or 16 for the
+// slices that even out the last round of workgroups (a quarter of the loader threads fetch them, every wave still
+// multiplies its 16 output channels).
+constexpr int cg_lds_floats(int tn) {
+    return CG_STAGES * 16 * tn * CG_PITCH > CG_BM * 16 * tn ? CG_STAGES * 16 * tn * CG_PITCH : CG_BM * 16 * tn;
+}
 template <int TN>
-__global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs p) {
+__device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_t m0, int64_t p0, float* lds, uint32_t* lds_tap) {
     constexpr int BM = CG_BM, BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
-    static_assert(BN % WAVE == 0, "a wave's loader units share their k-quad");
     constexpr int UNITS = BN * (BK / 4);                 // (position, k-quad) units of one tile
-    static_assert(UNITS % CG_THREADS == 0, "whole units per thread");
-    constexpr int B_PER_T = UNITS / CG_THREADS;
+    // whole waves of loader units share their k-quad (read once, on the scalar unit); a narrow slice has four
+    // k-quads per wave and only UNITS loader threads
+    constexpr bool UNIFORM_KQ = BN % WAVE == 0;
+    static_assert(UNITS % CG_THREADS == 0 || UNITS < CG_THREADS, "whole units per thread, or fewer units than threads");
+    constexpr int B_PER_T = UNITS >= CG_THREADS ? UNITS / CG_THREADS : 1;
     constexpr int STAGE = BN * PITCH;
-    constexpr int RED = BM * BN;                         // partial sums of k-split group 1
-    constexpr int LDS_FLOATS = CG_STAGES * STAGE > RED ? CG_STAGES * STAGE : RED;
-    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
-    // tap table: for every k = (c, r, s) the element offset of that tap relative to a
-    // position's top-left input pixel (low 27 bits) and the tap index r * KW + s (high 5 bits)
-    __shared__ __attribute__((aligned(16))) uint32_t lds_tap[CG_MAX_K];
+    static_assert(UNITS >= CG_THREADS || CG_STAGES * STAGE + (CG_STAGES - 1) * STAGE + 4 * CG_THREADS <= cg_lds_floats(4), "room for the idle threads' writes");
 
     const int tid = threadIdx.x;
+    const bool loader = UNITS >= CG_THREADS || tid < UNITS;   // whole waves
     const int lane = tid % WAVE, wave = tid / WAVE;
     const int li = lane % 16, lq = lane / 16;
     const int wm = wave % 4, ks = wave / 4;   // wave row, k-split group
@@ -272,11 +277,6 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
         const uint32_t t = rs - r * (uint32_t)p.KW;
         lds_tap[k] = (rs << 27) | (c * (uint32_t)(p.H * p.Wd) + r * (uint32_t)(p.dil_h * p.Wd) + t * (uint32_t)p.dil_w);
     }
-
-    const int64_t logical = xcd_remap(blockIdx.x, p.nwg);
-    int64_t tm, tn;
-    tile_coords(logical, p.tiles_m, p.tiles_p, p.group_m, tm, tn);
-    const int64_t m0 = tm * BM, p0 = tn * BN;
 
     // W operand of this lane: row oc (clamped), 4 floats at k = 32 kt + 16 ks + 4 lq
     int64_t am = m0 + 16 * wm + li;
@@ -290,7 +290,7 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
     uint32_t xbase = 0, tap_outside = 0xffffffffu;
     {
         const int64_t pp = p0 + p_local;
-        if (pp < p.P) {
+        if (pp < p.P && loader) {
             const uint32_t n = fdiv((uint32_t)pp, p.div_ohw);
             const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
             const uint32_t oy = fdiv(q, p.div_ow);
@@ -311,8 +311,13 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
     int kq[B_PER_T], b_lds[B_PER_T];
 #pragma unroll
     for (int it = 0; it < B_PER_T; ++it) {
-        kq[it] = __builtin_amdgcn_readfirstlane((tid + it * CG_THREADS) / BN);
+        kq[it] = (tid + it * CG_THREADS) / BN;
+        if constexpr (UNIFORM_KQ) kq[it] = __builtin_amdgcn_readfirstlane(kq[it]);
+        else kq[it] &= BK / 4 - 1;   // (threads that load nothing stay inside the table)
         b_lds[it] = p_local * PITCH + 4 * kq[it];
+        // a narrow slice keeps the step free of branches: the threads without a unit load nothing (every tap counts as
+        // outside) and write their zeros to a place of their own behind the three stages
+        if (!loader) b_lds[it] = CG_STAGES * STAGE + 4 * tid;
     }
 
     f32x4 acc[TN];
@@ -371,6 +376,7 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
         // gather loads, each memory instruction between MFMAs so that it never queues
         // behind the other waves' requests while the matrix pipe idles.
         constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
+        if constexpr (UNIFORM_KQ) {
         __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
         __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
         __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
@@ -385,6 +391,7 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
             __builtin_amdgcn_sched_group_barrier(VMEM_RD, 1, 0);
         }
         __builtin_amdgcn_sched_group_barrier(MFMA, 4 * TN, 0);
+        }
         __syncthreads();
     };
     static_assert(RING % 2 == 0 && RING % CG_STAGES == 0, "slot index fixes operand set and LDS buffer");
@@ -454,6 +461,24 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
                 p.Y[off] = conv_epilogue_tail1(v[r], p.epi, p.residual, off);
             }
         }
+    }
+}
+
+// TN: the whole tiles; workgroups past p.full_tiles take 16-position slices (TN = 1)
+template <int TN>
+__global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs p) {
+    __shared__ __attribute__((aligned(16))) float lds[cg_lds_floats(TN)];
+    // tap table: for every k = (c, r, s) the element offset of that tap relative to a
+    // position's top-left input pixel (low 27 bits) and the tap index r * KW + s (high 5 bits)
+    __shared__ __attribute__((aligned(16))) uint32_t lds_tap[CG_MAX_K];
+    if ((int64_t)blockIdx.x < p.full_tiles) {
+        const int64_t logical = xcd_remap(blockIdx.x, p.full_tiles);
+        int64_t tm, tn;
+        tile_coords(logical, p.tiles_m, p.tiles_p, p.group_m, tm, tn);
+        conv2d_f32_gather_tile<TN>(p, tm * CG_BM, tn * (16 * TN), lds, lds_tap);
+    } else {
+        const uint32_t q = blockIdx.x - (uint32_t)p.full_tiles, tiles_m = (uint32_t)p.tiles_m;
+        conv2d_f32_gather_tile<1>(p, (int64_t)(q % tiles_m) * CG_BM, p.p_full + 16 * (int64_t)(q / tiles_m), lds, lds_tap);
     }
 }
 
@@ -558,7 +583,25 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
         const int bn = wide ? 128 : 64;
         p.tiles_m = ceil_div(M, (int64_t)CG_BM);
         p.tiles_p = ceil_div(P, (int64_t)bn);
-        p.nwg = p.tiles_m * p.tiles_p;
+        p.full_tiles = p.tiles_m * p.tiles_p;
+        p.p_full = p.tiles_p * bn;
+        int64_t slices = 0;
+        // Narrow tiles in more than one round of workgroups, the last round less than half full (configuration 4:
+        // 1568 tiles on 512 places): the tiles of that round run as 16-position slices, four times as many
+        // workgroups of a quarter of the work each, so the places that would idle through a whole tile time
+        // share its work.
+        if (!wide && tuning().conv_tail != 0) {
+            const int64_t places = (int64_t)cus * 2, rem = p.full_tiles % places;
+            const int64_t tail_p = tuning().conv_tail > 0 ? tuning().conv_tail : rem / p.tiles_m;
+            const bool wanted = tuning().conv_tail > 0 || (p.full_tiles > places && rem > 0 && rem < places / 2);
+            if (wanted && tail_p > 0 && tail_p < p.tiles_p) {
+                p.tiles_p -= tail_p;
+                p.full_tiles = p.tiles_m * p.tiles_p;
+                p.p_full = p.tiles_p * bn;
+                slices = p.tiles_m * ceil_div(P - p.p_full, (int64_t)16);
+            }
+        }
+        p.nwg = p.full_tiles + slices;
         MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "conv2d: grid too large");
         if (wide) hipLaunchKernelGGL(conv2d_f32_gather_kernel<8>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
         else hipLaunchKernelGGL(conv2d_f32_gather_kernel<4>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);

@@ -485,6 +485,44 @@ def test_conv_residual_epilogue(shape, wshape, pads, strides, epi):
     assert lib.mi355x_conv2d_f32(*(args[:3] + args[4:-2] + [_lib.EPI_RESIDUAL, None])) == 1
 
 
+@pytest.mark.parametrize("shape, wshape, tail", [
+    ((3, 32, 20, 20), (64, 32, 3, 3), 2),      # 1200 positions: 18.75 tiles of 64 -> 16 whole tiles, 44 slices, the last one ragged
+    ((2, 64, 16, 16), (80, 64, 3, 3), 7),      # two tiles of output channels (the second partly filled), 1 whole tile per row of tiles
+    ((1, 32, 9, 9), (16, 32, 3, 3), 1)])       # 81 positions, odd: scalar stores in the slices
+@pytest.mark.parametrize("epi", [0, _lib.EPI_BIAS | _lib.EPI_RELU, _lib.EPI_BIAS | _lib.EPI_RESIDUAL | _lib.EPI_RELU_AFTER])
+def test_conv_last_round_as_slices(monkeypatch, shape, wshape, tail, epi):
+    """The convolution's last round of tiles run as 16-position slices (the library chooses that by the number of
+    tiles and CUs; here it is forced on small problems through MI355X_CONV_TAIL = number of position tiles to slice)."""
+    rng = np.random.default_rng(31 + tail)
+    x = rng.normal(size=shape).astype(np.float32)
+    w = (rng.normal(size=wshape) / np.sqrt(np.prod(wshape[1:]))).astype(np.float32)
+    b = rng.normal(size=wshape[0]).astype(np.float32)
+    pre = O.conv2d(x, w, b if epi & _lib.EPI_BIAS else None, strides=(1, 1), pads=(1, 1, 1, 1))
+    r = rng.normal(size=pre.shape).astype(np.float32)
+    expected = O.relu(pre) if epi & _lib.EPI_RELU else pre
+    expected = expected + r if epi & _lib.EPI_RESIDUAL else expected
+    expected = O.relu(expected) if epi & _lib.EPI_RELU_AFTER else expected
+    tx, tw, tb, tr = (torch.from_numpy(a).cuda() for a in (x, w, b, r))
+    lib = _lib.library()
+    args = lambda y: [tx.data_ptr(), tw.data_ptr(), tb.data_ptr() if epi & _lib.EPI_BIAS else None,
+                      tr.data_ptr() if epi & _lib.EPI_RESIDUAL else None, y.data_ptr(), *shape, wshape[0], 3, 3,
+                      _lib.i64_array([1, 1, 1, 1]), _lib.i64_array([1, 1]), _lib.i64_array([1, 1]), epi,
+                      torch.cuda.current_stream().cuda_stream]
+    results = []
+    for setting in (str(tail), "0"):
+        monkeypatch.setenv("MI355X_CONV_TAIL", setting)
+        lib.mi355x_reload_tuning()
+        y = torch.full(pre.shape, float("nan"), device="cuda")
+        assert lib.mi355x_conv2d_res_f32(*args(y)) == 0, lib.mi355x_last_error()
+        torch.cuda.synchronize()
+        results.append(y.cpu().numpy())
+    monkeypatch.delenv("MI355X_CONV_TAIL", raising=False)
+    lib.mi355x_reload_tuning()
+    assert rel_err(expected, results[0]) < FP32_REL_TOL
+    # a slice adds up the same products in the same order as the tile it stands in for
+    assert np.array_equal(results[0], results[1])
+
+
 def test_tasklet_fusion_programs_values():
     # tests/transformation/test_tasklet_fusion.py:9-60 of the reference: same inputs (ones, twos), same expectations
     from test_fusion import _tasklet_fusion_graphs
