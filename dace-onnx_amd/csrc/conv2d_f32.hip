@@ -298,7 +298,9 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
             const int iy0 = (int)oy * p.stride_h - p.pad_t;
             const int ix0 = (int)ox * p.stride_w - p.pad_l;
             // may point before the image inside the pad: only ever added to tap offsets that bring it back
-            xbase = (uint32_t)(((int)n * p.C * p.H * p.Wd + iy0 * p.Wd + ix0) * 4);
+            // relative to pad_t rows and pad_l pixels before X, so that it is never negative: it is the bounds-checked
+            // part of the address (the tap offset goes into the load's scalar offset, which is not checked)
+            xbase = (uint32_t)(((int)n * p.C * p.H * p.Wd + (iy0 + p.pad_t) * p.Wd + ix0 + p.pad_l) * 4);
             tap_outside = 0;
             for (int r = 0; r < p.KH; ++r)
                 for (int t = 0; t < p.KW; ++t) {
@@ -335,18 +337,31 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     };
     auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt) __attribute__((always_inline)) {
         const int k0 = (kt < last_tile ? kt : last_tile) * BK;
-        // X as a raw buffer: an offset with bit 31 set is out of range and loads 0.0f, so a
-        // padded tap costs no branch and no select (X is smaller than 2 GiB, checked at launch)
-        const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.X), 0, p.x_bytes, 0x00020000);
+        // X as a raw buffer of 2^31 - 1 bytes: an offset with bit 31 set is out of range and loads 0.0f, so a
+        // padded tap costs no branch and no select; every other tap lies inside X (which, with its leading
+        // pad, is smaller than 2 GiB: checked at launch)
+        const int lead = (p.pad_t * p.Wd + p.pad_l) * 4;   // bytes of the (virtual) pad rows and pixels before X
+        const __amdgpu_buffer_rsrc_t x_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(p.X)) - lead, 0, 0x7fffffff, 0x00020000);
 #pragma unroll
         for (int it = 0; it < B_PER_T; ++it) {
             // the four taps of this unit's k-quad: one broadcast read (same address in every lane)
             const u32x4 taps = *reinterpret_cast<const u32x4*>(lds_tap + k0 + 4 * kq[it]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const uint32_t off = xbase + ((taps[e] & 0x07ffffffu) << 2);
-                const uint32_t outside = (tap_outside >> (taps[e] >> 27)) & 1u;
-                dst[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(off | (outside << 31)), 0, 0));
+                // Vector instructions take their time out of the matrix pipe's (measured: 3 to 5 cycles each, whatever
+                // the number of waves), so what is the same for the whole wave is computed on the scalar unit: the
+                // tap's offset travels as the load's scalar offset, its index selects the lane's pad bit with one
+                // bit-field extract, and one shift-or marks the padded lanes out of range.
+                if constexpr (UNIFORM_KQ) {
+                    const uint32_t tap = (uint32_t)__builtin_amdgcn_readfirstlane((int)taps[e]);
+                    const uint32_t outside = __builtin_amdgcn_ubfe(tap_outside, tap >> 27, 1u);
+                    dst[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(xbase | (outside << 31)), (int)((tap & 0x07ffffffu) << 2), 0));
+                } else {
+                    const uint32_t off = xbase + ((taps[e] & 0x07ffffffu) << 2);
+                    const uint32_t outside = (tap_outside >> (taps[e] >> 27)) & 1u;
+                    dst[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)(off | (outside << 31)), 0, 0));
+                }
             }
         }
     };
@@ -570,7 +585,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
     p.group_m = 1;
     // K a multiple of the 32-k tile and 16-byte aligned W rows: the gather kernel
     if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && C * H * Wd < ((int64_t)1 << 27) &&
-        N * C * H * Wd < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
+        N * C * H * Wd + pads[0] * Wd + pads[1] < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
         p.x_bytes = (int)(N * C * H * Wd * 4);
         // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
         // at the same rate, so the choice is the number of rounds times the tile width; ties go
