@@ -549,7 +549,8 @@ class MI355XBatchNormalization(ONNXForward):
 
 @op_implementation(op="MatMulInteger", name=IMPLEMENTATION_NAME)
 class MI355XMatMulInteger(ONNXForward):
-    """8-bit x 8-bit -> int32 on int8 MFMA, bit-exact; operands int8 or uint8 (independently), zero
+    """8-bit x 8-bit -> int32 on int8 MFMA, bit-exact against the ONNX formula in 64-bit integers (parity with the
+    reference unpinned: it has no implementation of its own); operands int8 or uint8 (independently), zero
     points read on the device: absent, one value, one per row of A or one per column of B. A may be
     a stack of matrices against a 2-D B (the stack is folded into M). The reference can only run this
     node through ONNX Runtime (onnx_op.py:686-687)."""

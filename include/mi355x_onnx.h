@@ -141,7 +141,9 @@ int mi355x_batchnorm_f32(const float* X, const float* scale, const float* B, con
                          const float* var, float* Y, int64_t N, int64_t C, int64_t HW, float eps,
                          void* stream);
 
-/* ONNX MatMulInteger (opset 10), 8-bit operands -> int32 on int8 MFMA, bit-exact.
+/* ONNX MatMulInteger (opset 10), 8-bit operands -> int32 on int8 MFMA, bit-exact against the formula below
+ * evaluated in 64-bit integers (wrapped to 32 bits); parity with the reference is unpinned: it has no
+ * implementation of its own to compare with.
  *   Y[m,n] = sum_k (A[m,k] - a_zero_point[m]) * (B[k,n] - b_zero_point[n])
  * The reference has no expansion of its own for this node: the generated class
  * (daceml/onnx/nodes/onnx_op.py:623-640, built from the ONNX schema: T1, T2 in
