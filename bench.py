@@ -157,8 +157,11 @@ def main():
     if mode == "auto":
         # a graph replay has one launch but a few microseconds between replays; host-issued
         # launches have none of that but need the host to stay ahead of the GPU
-        timed(eager_step, 5), timed(compiled.replay, 5)
-        t_eager, t_graph = timed(eager_step, args.warmup), timed(compiled.replay, args.warmup)
+        # (compared once the core clock is up, over enough steps for the difference of a few per cent to show)
+        warm_up(compiled.replay, WARM_MS)
+        n_compare = max(args.warmup, 200)
+        t_eager, t_graph = timed(eager_step, n_compare), timed(compiled.replay, n_compare)
+        t_eager, t_graph = min(t_eager, timed(eager_step, n_compare)), min(t_graph, timed(compiled.replay, n_compare))
         mode, step = ("eager", eager_step) if t_eager < t_graph else ("graph", compiled.replay)
     else:
         timed(step, args.warmup)
