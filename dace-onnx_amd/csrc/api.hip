@@ -33,6 +33,13 @@ static Tuning g_tuning;
 static std::atomic<bool> g_tuning_valid{false};
 static std::mutex g_tuning_mutex;
 
+#ifdef MI355X_WG_TRACE
+unsigned long long* trace_buffer() {
+    const char* v = getenv("MI355X_WG_TRACE_BUFFER");
+    return v && *v ? reinterpret_cast<unsigned long long*>(strtoull(v, nullptr, 10)) : nullptr;
+}
+#endif
+
 static int env_int(const char* name, int fallback) {
     const char* v = getenv(name);
     return v && *v ? atoi(v) : fallback;

@@ -32,6 +32,35 @@ struct Tuning {
 const Tuning& tuning();
 int device_cus();
 
+// Workgroup trace, compiled in only with -DMI355X_WG_TRACE (`make trace` builds libmi355x_onnx_trace.so): the contraction
+// kernels stamp the wall clock (100 MHz) at the start of a workgroup, at the first and after the last step of its main
+// loop and at its end, plus the hardware id of the CU it runs on, into the buffer whose device address the environment
+// variable MI355X_WG_TRACE_BUFFER holds (8 x 64-bit words per workgroup; unset: no stamps). The normal build carries
+// neither the argument nor the code.
+#ifdef MI355X_WG_TRACE
+#define MI355X_TRACE_MEMBER unsigned long long* trace;
+#define MI355X_TRACE_INIT(args) (args).trace = ::mi355x::trace_buffer()
+#define MI355X_TRACE_STAMP(args, slot)                                                          \
+    do {                                                                                        \
+        if ((args).trace && threadIdx.x == 0) (args).trace[8 * blockIdx.x + (slot)] = wall_clock64(); \
+    } while (0)
+#define MI355X_TRACE_HWID(args)                                                                 \
+    do {                                                                                        \
+        if ((args).trace && threadIdx.x == 0) {                                                 \
+            unsigned hw_, xcc_;                                                                 \
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_));                   \
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_));                 \
+            (args).trace[8 * blockIdx.x + 4] = ((unsigned long long)xcc_ << 32) | hw_;          \
+        }                                                                                       \
+    } while (0)
+unsigned long long* trace_buffer();
+#else
+#define MI355X_TRACE_MEMBER
+#define MI355X_TRACE_INIT(args) do {} while (0)
+#define MI355X_TRACE_STAMP(args, slot) do {} while (0)
+#define MI355X_TRACE_HWID(args) do {} while (0)
+#endif
+
 // ---- device side -------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));

@@ -74,6 +74,7 @@ struct ConvArgs {
     int x_bytes;    // size of X (gather kernel only; below 2^31)
     // gather kernel: the first full_tiles workgroups take whole tiles, the rest 16-position slices from p_full on
     int64_t full_tiles, p_full;
+    MI355X_TRACE_MEMBER
 };
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool VEC_W>
@@ -254,7 +255,7 @@ constexpr int cg_lds_floats(int tn) {
 }
 template <int TN>
 __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_t m0, int64_t p0, float* lds, uint32_t* lds_tap) {
-    constexpr int BM = CG_BM, BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
+    constexpr int BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
     constexpr int UNITS = BN * (BK / 4);                 // (position, k-quad) units of one tile
     // whole waves of loader units share their k-quad (read once, on the scalar unit); a narrow slice has four
     // k-quads per wave and only UNITS loader threads
@@ -264,6 +265,8 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     constexpr int STAGE = BN * PITCH;
     static_assert(UNITS >= CG_THREADS || CG_STAGES * STAGE + (CG_STAGES - 1) * STAGE + 4 * CG_THREADS <= cg_lds_floats(4), "room for the idle threads' writes");
 
+    MI355X_TRACE_STAMP(p, 0);
+    MI355X_TRACE_HWID(p);
     const int tid = threadIdx.x;
     const bool loader = UNITS >= CG_THREADS || tid < UNITS;   // whole waves
     const int lane = tid % WAVE, wave = tid / WAVE;
@@ -426,6 +429,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     // Whole groups of RING steps run without a branch inside the loop (with guards in the body the
     // compiler's wait-count analysis drains every outstanding load at the loop header); the at most
     // RING - 1 remaining steps follow, guarded.
+    MI355X_TRACE_STAMP(p, 1);
     int kt0 = 0;
     for (; kt0 + RING <= ktiles; kt0 += RING) {
         cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) { tile_step(r_tag, kt0 + decltype(r_tag)::value); });
@@ -435,6 +439,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         if (kt < ktiles) tile_step(r_tag, kt);  // uniform
     });
 
+    MI355X_TRACE_STAMP(p, 2);
     // k-split group 1 hands its partial sums to group 0 through LDS
     {
         f32x4* red = reinterpret_cast<f32x4*>(lds);
@@ -477,6 +482,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
             }
         }
     }
+    MI355X_TRACE_STAMP(p, 3);
 }
 
 // TN: the whole tiles; workgroups past p.full_tiles take 16-position slices (TN = 1)
@@ -565,6 +571,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
                    "conv2d: tensor too large for 32-bit gather offsets");
 
     ConvArgs p;
+    MI355X_TRACE_INIT(p);
     p.X = X; p.W = W; p.bias = bias; p.Y = Y; p.residual = residual;
     p.N = (int)N; p.C = (int)C; p.H = (int)H; p.Wd = (int)Wd; p.M = (int)M; p.KH = (int)KH; p.KW = (int)KW;
     p.OH = (int)OH; p.OW = (int)OW; p.OHW = (int)(OH * OW);

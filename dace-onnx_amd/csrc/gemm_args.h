@@ -17,6 +17,7 @@ struct GemmArgs {
     int group_m;  // tile walk order, see tile_coords
     float alpha;
     int epi;
+    MI355X_TRACE_MEMBER
 };
 
 // GEMM with both operands contiguous along k (gemm_f32_nt.hip). Returns false when

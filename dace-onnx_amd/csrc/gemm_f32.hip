@@ -214,6 +214,7 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     MI355X_REQUIRE(c_strides[2] >= N || M == 1, "gemm: C row stride %lld < N %lld", (long long)c_strides[2], (long long)N);
 
     GemmArgs p;
+    MI355X_TRACE_INIT(p);
     p.A = A; p.B = B; p.C = C; p.bias = bias; p.residual = residual;
     p.batch = batch; p.batch1 = batch1; p.M = M; p.N = N; p.K = K;
     p.a_sb0 = a_strides[0]; p.a_sb1 = a_strides[1]; p.a_sm = a_strides[2]; p.a_sk = a_strides[3];

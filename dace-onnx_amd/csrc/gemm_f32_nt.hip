@@ -68,6 +68,8 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     const int lane = tid % WAVE, wave = tid / WAVE;
     const int li = lane % 16, lq = lane / 16;
     const int wm = wave % WAVES_M, ks = wave / WAVES_M;   // wave row, k-split group
+    MI355X_TRACE_STAMP(p, 0);
+    MI355X_TRACE_HWID(p);
 
     const int64_t logical = xcd_remap(blockIdx.x, p.nwg);
     const uint32_t tiles_per_batch = (uint32_t)(p.tiles_m * p.tiles_n);
@@ -208,6 +210,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     store_b(rb[1], 1);
     __syncthreads();
     read_b(bf[0], 0, 0);
+    MI355X_TRACE_STAMP(p, 1);
 
     // One code path for every tile: near the end of K the look-aheads are not switched
     // off but clamped to the last tile (they re-read data that is already in cache and
@@ -221,6 +224,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         });
     }
 
+    MI355X_TRACE_STAMP(p, 2);
     // k-split group 1 hands its partial sums to group 0 through LDS
     if constexpr (KSPLIT == 2) {
         f32x4* red = reinterpret_cast<f32x4*>(lds);
@@ -255,6 +259,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         else if (R) v += *reinterpret_cast<const f32x4*>(R + m * p.r_sm + n);
         *reinterpret_cast<f32x4*>(C + m * p.c_sm + n) = v;
     }
+    MI355X_TRACE_STAMP(p, 3);
 }
 
 // The caller guarantees: 16-byte aligned operands, a_sk == b_sk == 1, every stride

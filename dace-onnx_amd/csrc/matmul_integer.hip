@@ -28,6 +28,7 @@ struct MMIArgs {
     int a_unsigned, b_unsigned;
     int64_t tiles_m, tiles_n, nwg;
     int group_m;  // tile walk order, see tile_coords
+    MI355X_TRACE_MEMBER
 };
 
 typedef int i32x2 __attribute__((ext_vector_type(2)));
@@ -311,6 +312,8 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     const int wm = wave / 2, wn = wave % 2;
     const int wm0 = wm * 64, wn0 = wn * 64;
 
+    MI355X_TRACE_STAMP(p, 0);
+    MI355X_TRACE_HWID(p);
     const int ktiles = (int)(p.K / BK);
     // tiles of this workgroup: blockIdx.x + i * gridDim.x (gridDim.x is a multiple of 8 or the whole tile
     // count, so all of them run on this workgroup's XCD and xcd_remap keeps them in its slab)
@@ -550,6 +553,7 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
         MI355X_WAIT_VMCNT(0);
     }
     __syncthreads();
+    MI355X_TRACE_STAMP(p, 1);   // the first operands are in LDS
     read_frags(0, 0, 0);
 
     int kt = 0, tile_i = 0, stage = 0;
@@ -581,7 +585,12 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
         __syncthreads();
         stage = stage1;
     }
+    MI355X_TRACE_STAMP(p, 2);
     if (pending) finish_tile(tile_i - 1);
+#ifdef MI355X_WG_TRACE
+    if (p.trace) MI355X_WAIT_VMCNT(0);   // slot 3: the last store is acknowledged
+#endif
+    MI355X_TRACE_STAMP(p, 3);
 }
 
 template <bool ZP>
@@ -624,6 +633,7 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
     auto al = [](const void* q, int a) { return (reinterpret_cast<uintptr_t>(q) & (a - 1)) == 0; };
     hipStream_t st = static_cast<hipStream_t>(stream);
     p.group_m = 1;
+    MI355X_TRACE_INIT(p);
     const Tuning& tune = tuning();
     const int cus = device_cus();
     // 16-byte transfers of A rows and B rows; a tile's 128 rows of Y are addressed with 31-bit byte offsets
