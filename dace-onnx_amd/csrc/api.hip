@@ -55,6 +55,7 @@ static void parse_tuning(Tuning& t) {
     t.conv_config = c && c[0] >= '0' && c[0] <= '9' ? c[0] - '0' : -1;
     t.conv_gather_bn = env_int("MI355X_CONV_GATHER_BN", 0);
     t.conv_tail = env_int("MI355X_CONV_TAIL", -1);
+    t.conv_static_taps = env_int("MI355X_CONV_STATIC_TAPS", 1);
     t.mmi_generic = getenv("MI355X_MMI_GENERIC") != nullptr;
     t.mmi_wgs_per_cu = env_int("MI355X_MMI_WGS_PER_CU", 0);
 }

@@ -253,13 +253,27 @@ __device__ __forceinline__ void cg_static_for(F&& f) {
 constexpr int cg_lds_floats(int tn) {
     return CG_STAGES * 16 * tn * CG_PITCH > CG_BM * 16 * tn ? CG_STAGES * 16 * tn * CG_PITCH : CG_BM * 16 * tn;
 }
-template <int TN>
+constexpr int cg_gcd(int a, int b) { return b == 0 ? a : cg_gcd(b, a % b); }
+// TAPS: 0, or KH * KW when C % 32 == 0 (K a whole number of windows of 32 channels). Then the gather needs no tap
+// table and no vector arithmetic. With k = TAPS c + rs, the unit of a wave that covers k = 32 kt + 4 kq + e meets
+// the taps in a pattern that repeats every WIN = TAPS / gcd(32, TAPS) steps: write 4 kq = TAPS a + rot and
+// 32 i + e = TAPS n + j for step i of a window; then rs = (j + rot) mod TAPS and c = 32 window + a + n + [j + rot >= TAPS].
+// rot is fixed for a wave, so the lane keeps, for j = 0 .. TAPS - 1, the byte offset of tap (j + rot) mod TAPS
+// from its position's first pixel, plus one channel where j + rot wraps, with bit 31 set where that tap is
+// padding: the load of (i, e) takes register j (known at compile time) as its vector offset and the running
+// channel offset (a + 32 window + n) H W 4, kept on the scalar unit, as its scalar offset.
+template <int TN, int TAPS = 0>
 __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_t m0, int64_t p0, float* lds, uint32_t* lds_tap) {
     constexpr int BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
+    constexpr bool STATIC_TAPS = TAPS > 0;
+    constexpr int WIN = STATIC_TAPS ? TAPS / cg_gcd(BK, TAPS ? TAPS : 1) : 1;        // steps per window
+    constexpr int UNROLL = RING * WIN / cg_gcd(RING, WIN);                           // slot and window position both fixed
+    constexpr int NTAP = STATIC_TAPS ? TAPS : 1;
     constexpr int UNITS = BN * (BK / 4);                 // (position, k-quad) units of one tile
     // whole waves of loader units share their k-quad (read once, on the scalar unit); a narrow slice has four
     // k-quads per wave and only UNITS loader threads
     constexpr bool UNIFORM_KQ = BN % WAVE == 0;
+    static_assert(!STATIC_TAPS || UNIFORM_KQ, "compile-time taps need one k-quad per wave");
     static_assert(UNITS % CG_THREADS == 0 || UNITS < CG_THREADS, "whole units per thread, or fewer units than threads");
     constexpr int B_PER_T = UNITS >= CG_THREADS ? UNITS / CG_THREADS : 1;
     constexpr int STAGE = BN * PITCH;
@@ -273,12 +287,14 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     const int li = lane % 16, lq = lane / 16;
     const int wm = wave % 4, ks = wave / 4;   // wave row, k-split group
 
-    for (int k = tid; k < p.K; k += CG_THREADS) {
-        const uint32_t c = fdiv((uint32_t)k, p.div_khw);
-        const uint32_t rs = (uint32_t)k - c * (uint32_t)(p.KH * p.KW);
-        const uint32_t r = fdiv(rs, p.div_kw);
-        const uint32_t t = rs - r * (uint32_t)p.KW;
-        lds_tap[k] = (rs << 27) | (c * (uint32_t)(p.H * p.Wd) + r * (uint32_t)(p.dil_h * p.Wd) + t * (uint32_t)p.dil_w);
+    if constexpr (!STATIC_TAPS) {
+        for (int k = tid; k < p.K; k += CG_THREADS) {
+            const uint32_t c = fdiv((uint32_t)k, p.div_khw);
+            const uint32_t rs = (uint32_t)k - c * (uint32_t)(p.KH * p.KW);
+            const uint32_t r = fdiv(rs, p.div_kw);
+            const uint32_t t = rs - r * (uint32_t)p.KW;
+            lds_tap[k] = (rs << 27) | (c * (uint32_t)(p.H * p.Wd) + r * (uint32_t)(p.dil_h * p.Wd) + t * (uint32_t)p.dil_w);
+        }
     }
 
     // W operand of this lane: row oc (clamped), 4 floats at k = 32 kt + 16 ks + 4 lq
@@ -291,6 +307,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     // falls outside the image (pad) for this position. KH * KW <= 32 is a launch precondition.
     const int p_local = tid % BN;
     uint32_t xbase = 0, tap_outside = 0xffffffffu;
+    int iy0 = 0, ix0 = 0;
     {
         const int64_t pp = p0 + p_local;
         if (pp < p.P && loader) {
@@ -298,8 +315,8 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
             const uint32_t q = (uint32_t)pp - n * (uint32_t)p.OHW;
             const uint32_t oy = fdiv(q, p.div_ow);
             const uint32_t ox = q - oy * (uint32_t)p.OW;
-            const int iy0 = (int)oy * p.stride_h - p.pad_t;
-            const int ix0 = (int)ox * p.stride_w - p.pad_l;
+            iy0 = (int)oy * p.stride_h - p.pad_t;
+            ix0 = (int)ox * p.stride_w - p.pad_l;
             // may point before the image inside the pad: only ever added to tap offsets that bring it back
             // relative to pad_t rows and pad_l pixels before X, so that it is never negative: it is the bounds-checked
             // part of the address (the tap offset goes into the load's scalar offset, which is not checked)
@@ -324,6 +341,24 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         // outside) and write their zeros to a place of their own behind the three stages
         if (!loader) b_lds[it] = CG_STAGES * STAGE + 4 * tid;
     }
+    // compile-time taps: the lane's offsets in the wave's rotation, and the wave's running channel offset
+    const uint32_t hw4 = (uint32_t)(p.H * p.Wd) * 4u;
+    const uint32_t soff_safe = (uint32_t)(p.C - 2) * hw4;   // for the look-aheads past the last step: inside X with or without the wrap
+    uint32_t vtap[B_PER_T][NTAP], soff[B_PER_T];
+    if constexpr (STATIC_TAPS) {
+#pragma unroll
+        for (int it = 0; it < B_PER_T; ++it) {
+            const uint32_t a = (uint32_t)(4 * kq[it]) / (uint32_t)TAPS, rot = (uint32_t)(4 * kq[it]) - a * (uint32_t)TAPS;
+            soff[it] = a * hw4;
+#pragma unroll
+            for (int j = 0; j < TAPS; ++j) {
+                const uint32_t jj = (uint32_t)j + rot, wrap = jj >= (uint32_t)TAPS ? 1u : 0u, rs = jj - wrap * (uint32_t)TAPS;
+                const uint32_t r = fdiv(rs, p.div_kw), t = rs - r * (uint32_t)p.KW;
+                const uint32_t outside = (tap_outside >> rs) & 1u;
+                vtap[it][j] = (xbase + (r * (uint32_t)(p.dil_h * p.Wd) + t * (uint32_t)p.dil_w) * 4u + wrap * hw4) | (outside << 31);
+            }
+        }
+    }
 
     f32x4 acc[TN];
 #pragma unroll
@@ -338,7 +373,8 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     auto load_a = [&](f32x4& dst, int kt) __attribute__((always_inline)) {
         dst = *reinterpret_cast<const f32x4*>(a_ptr + (int64_t)(kt < last_tile ? kt : last_tile) * BK);
     };
-    auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt) __attribute__((always_inline)) {
+    auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt, auto i_tag) __attribute__((always_inline)) {
+        constexpr int I = decltype(i_tag)::value;   // the step's place in its window (compile-time taps)
         const int k0 = (kt < last_tile ? kt : last_tile) * BK;
         // X as a raw buffer of 2^31 - 1 bytes: an offset with bit 31 set is out of range and loads 0.0f, so a
         // padded tap costs no branch and no select; every other tap lies inside X (which, with its leading
@@ -346,6 +382,20 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         const int lead = (p.pad_t * p.Wd + p.pad_l) * 4;   // bytes of the (virtual) pad rows and pixels before X
         const __amdgpu_buffer_rsrc_t x_rsrc =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(p.X)) - lead, 0, 0x7fffffff, 0x00020000);
+        if constexpr (STATIC_TAPS) {
+#pragma unroll
+            for (int it = 0; it < B_PER_T; ++it) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    constexpr int S = BK * I, NEXT = BK * (I + 1);
+                    const int s_now = S + e, s_next = e < 3 ? S + e + 1 : NEXT;
+                    const uint32_t so = kt <= last_tile ? soff[it] : soff_safe;
+                    dst[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)vtap[it][s_now % NTAP], (int)so, 0));
+                    soff[it] += (uint32_t)(s_next / NTAP - s_now / NTAP) * hw4;
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int it = 0; it < B_PER_T; ++it) {
             // the four taps of this unit's k-quad: one broadcast read (same address in every lane)
@@ -378,10 +428,10 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
             dst[j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
     };
 
-    auto tile_step = [&](auto r_tag, int kt) __attribute__((always_inline)) {
-        constexpr int r = decltype(r_tag)::value;
+    auto tile_step = [&](auto u_tag, int kt) __attribute__((always_inline)) {
+        constexpr int r = decltype(u_tag)::value % RING;
         constexpr int cur = r & 1;  // RING is even: tile parity == slot parity
-        load_b(rb[r], kt + RING);                           // slot r went to LDS two steps ago
+        load_b(rb[r], kt + RING, std::integral_constant<int, (decltype(u_tag)::value + RING) % WIN>{});   // slot r went to LDS two steps ago
         load_a(ra[(r + RING - 1) % RING], kt + RING - 1);   // operand consumed in the previous step
         store_b(rb[(r + 2) % RING], (r + 2) % CG_STAGES);   // tile kt + 2
         read_b(bf[cur ^ 1], (r + 1) % CG_STAGES);           // tile kt + 1, visible since the last barrier
@@ -397,7 +447,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         if constexpr (UNIFORM_KQ) {
         __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
         __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
-        __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
+        if constexpr (!STATIC_TAPS) __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
@@ -417,8 +467,10 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
 #pragma unroll
     for (int r = 0; r < RING; ++r) load_a(ra[r], r);  // tiles beyond the last are clamped: no branch
     __syncthreads();  // tap table complete
-#pragma unroll
-    for (int r = 0; r < RING; ++r) load_b(rb[r], r);
+    cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) {
+        constexpr int r = decltype(r_tag)::value;
+        load_b(rb[r], r, std::integral_constant<int, r % WIN>{});
+    });
     store_b(rb[0], 0);
     store_b(rb[1], 1);
     __syncthreads();
@@ -431,12 +483,12 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     // RING - 1 remaining steps follow, guarded.
     MI355X_TRACE_STAMP(p, 1);
     int kt0 = 0;
-    for (; kt0 + RING <= ktiles; kt0 += RING) {
-        cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) { tile_step(r_tag, kt0 + decltype(r_tag)::value); });
+    for (; kt0 + UNROLL <= ktiles; kt0 += UNROLL) {
+        cg_static_for<UNROLL>([&](auto u_tag) __attribute__((always_inline)) { tile_step(u_tag, kt0 + decltype(u_tag)::value); });
     }
-    cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) {
-        const int kt = kt0 + decltype(r_tag)::value;
-        if (kt < ktiles) tile_step(r_tag, kt);  // uniform
+    cg_static_for<UNROLL>([&](auto u_tag) __attribute__((always_inline)) {
+        const int kt = kt0 + decltype(u_tag)::value;
+        if (kt < ktiles) tile_step(u_tag, kt);  // uniform
     });
 
     MI355X_TRACE_STAMP(p, 2);
@@ -486,7 +538,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
 }
 
 // TN: the whole tiles; workgroups past p.full_tiles take 16-position slices (TN = 1)
-template <int TN>
+template <int TN, int TAPS>
 __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs p) {
     __shared__ __attribute__((aligned(16))) float lds[cg_lds_floats(TN)];
     // tap table: for every k = (c, r, s) the element offset of that tap relative to a
@@ -496,7 +548,7 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
         const int64_t logical = xcd_remap(blockIdx.x, p.full_tiles);
         int64_t tm, tn;
         tile_coords(logical, p.tiles_m, p.tiles_p, p.group_m, tm, tn);
-        conv2d_f32_gather_tile<TN>(p, tm * CG_BM, tn * (16 * TN), lds, lds_tap);
+        conv2d_f32_gather_tile<TN, TAPS>(p, tm * CG_BM, tn * (16 * TN), lds, lds_tap);
     } else {
         const uint32_t q = blockIdx.x - (uint32_t)p.full_tiles, tiles_m = (uint32_t)p.tiles_m;
         conv2d_f32_gather_tile<1>(p, (int64_t)(q % tiles_m) * CG_BM, p.p_full + 16 * (int64_t)(q / tiles_m), lds, lds_tap);
@@ -592,7 +644,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
     p.group_m = 1;
     // K a multiple of the 32-k tile and 16-byte aligned W rows: the gather kernel
     if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && C * H * Wd < ((int64_t)1 << 27) &&
-        N * C * H * Wd + pads[0] * Wd + pads[1] < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
+        N * C * H * Wd + pads[0] * Wd + pads[1] + H * Wd < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
         p.x_bytes = (int)(N * C * H * Wd * 4);
         // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
         // at the same rate, so the choice is the number of rounds times the tile width; ties go
@@ -625,8 +677,18 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
         }
         p.nwg = p.full_tiles + slices;
         MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "conv2d: grid too large");
-        if (wide) hipLaunchKernelGGL(conv2d_f32_gather_kernel<8>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
-        else hipLaunchKernelGGL(conv2d_f32_gather_kernel<4>, dim3((unsigned)p.nwg), dim3(CG_THREADS), 0, st, p);
+        // 3 x 3 and 1 x 1 filters over whole windows of 32 channels: taps known at compile time
+        const int taps = (C % 32 == 0 && (KH * KW == 9 || KH * KW == 1) && tuning().conv_static_taps) ? (int)(KH * KW) : 0;
+        const dim3 g((unsigned)p.nwg), b(CG_THREADS);
+        if (wide) {
+            if (taps == 9) hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 9>), g, b, 0, st, p);
+            else if (taps == 1) hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 1>), g, b, 0, st, p);
+            else hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 0>), g, b, 0, st, p);
+        } else {
+            if (taps == 9) hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 9>), g, b, 0, st, p);
+            else if (taps == 1) hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 1>), g, b, 0, st, p);
+            else hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 0>), g, b, 0, st, p);
+        }
         return check_launch("conv2d_f32_gather_kernel");
     }
     const int cfg = choose_conv_tile(M, P, cus);

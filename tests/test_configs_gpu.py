@@ -523,6 +523,44 @@ def test_conv_last_round_as_slices(monkeypatch, shape, wshape, tail, epi):
     assert np.array_equal(results[0], results[1])
 
 
+@pytest.mark.parametrize("shape, wshape, strides, pads, dilations, gather_bn", [
+    ((2, 32, 12, 12), (64, 32, 3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 64),     # one window of 9 steps
+    ((1, 64, 14, 14), (48, 64, 3, 3), (1, 1), (1, 1, 1, 1), (1, 1), 128),    # the unrolled 18 steps once, wide tiles
+    ((2, 96, 11, 13), (64, 96, 3, 3), (2, 2), (1, 0, 2, 1), (1, 1), 64),     # 27 steps: 18 + a remainder of 9; stride 2, uneven pads
+    ((1, 160, 9, 9), (32, 160, 3, 3), (1, 1), (2, 2, 2, 2), (2, 2), 128),    # 45 steps, dilation 2
+    ((1, 32, 10, 7), (16, 32, 1, 9), (1, 1), (0, 4, 0, 4), (1, 1), 64),      # nine taps in one row
+    ((3, 64, 9, 9), (64, 64, 1, 1), (1, 1), (0, 0, 0, 0), (1, 1), 64),       # 1 x 1
+    ((2, 224, 8, 8), (40, 224, 1, 1), (2, 2), (0, 0, 0, 0), (1, 1), 128)])   # 1 x 1, stride 2, 7 steps
+def test_conv_taps_known_at_compile_time(monkeypatch, shape, wshape, strides, pads, dilations, gather_bn):
+    """3 x 3 and 1 x 1 filters over a multiple of 32 channels take a gather whose tap offsets are compile-time
+    register choices plus a scalar channel offset; MI355X_CONV_STATIC_TAPS=0 sends the same call through the tap
+    table. Both add up the same products in the same order."""
+    rng = np.random.default_rng(77 + shape[1])
+    x = rng.normal(size=shape).astype(np.float32)
+    w = (rng.normal(size=wshape) / np.sqrt(np.prod(wshape[1:]))).astype(np.float32)
+    b = rng.normal(size=wshape[0]).astype(np.float32)
+    expected = O.relu(O.conv2d(x, w, b, strides=strides, pads=pads, dilations=dilations))
+    tx, tw, tb = (torch.from_numpy(a).cuda() for a in (x, w, b))
+    lib = _lib.library()
+    monkeypatch.setenv("MI355X_CONV_GATHER_BN", str(gather_bn))
+    results = []
+    for setting in ("1", "0"):
+        monkeypatch.setenv("MI355X_CONV_STATIC_TAPS", setting)
+        lib.mi355x_reload_tuning()
+        y = torch.full(expected.shape, float("nan"), device="cuda")
+        status = lib.mi355x_conv2d_f32(tx.data_ptr(), tw.data_ptr(), tb.data_ptr(), y.data_ptr(), *shape, wshape[0], wshape[2], wshape[3],
+                                       _lib.i64_array(pads), _lib.i64_array(strides), _lib.i64_array(dilations),
+                                       _lib.EPI_BIAS | _lib.EPI_RELU, torch.cuda.current_stream().cuda_stream)
+        assert status == 0, lib.mi355x_last_error()
+        torch.cuda.synchronize()
+        results.append(y.cpu().numpy())
+    monkeypatch.delenv("MI355X_CONV_STATIC_TAPS", raising=False)
+    monkeypatch.delenv("MI355X_CONV_GATHER_BN", raising=False)
+    lib.mi355x_reload_tuning()
+    assert rel_err(expected, results[0]) < FP32_REL_TOL
+    assert np.array_equal(results[0], results[1])
+
+
 def test_tasklet_fusion_programs_values():
     # tests/transformation/test_tasklet_fusion.py:9-60 of the reference: same inputs (ones, twos), same expectations
     from test_fusion import _tasklet_fusion_graphs
