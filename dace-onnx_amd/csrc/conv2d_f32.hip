@@ -467,12 +467,15 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
 #pragma unroll
     for (int r = 0; r < RING; ++r) load_a(ra[r], r);  // tiles beyond the last are clamped: no branch
     __syncthreads();  // tap table complete
+    MI355X_TRACE_STAMP(p, 5);
     cg_static_for<RING>([&](auto r_tag) __attribute__((always_inline)) {
         constexpr int r = decltype(r_tag)::value;
         load_b(rb[r], r, std::integral_constant<int, r % WIN>{});
     });
+    MI355X_TRACE_STAMP(p, 6);
     store_b(rb[0], 0);
     store_b(rb[1], 1);
+    MI355X_TRACE_STAMP(p, 7);
     __syncthreads();
     read_b(bf[0], 0);
 

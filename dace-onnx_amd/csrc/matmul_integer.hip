@@ -289,9 +289,12 @@ constexpr int MMF_A_STAGE = MMF_BM * MMF_BK, MMF_B_STAGE = MMF_BK * MMF_BN, MMF_
 __device__ __forceinline__ i32x2 lds_read_tr8(const uint8_t* p) {
     return __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p));
 }
-// 16 bytes per lane from global memory into LDS at lds_addr + 16 * lane (lds_addr is wave-uniform)
-__device__ __forceinline__ void global_to_lds_16(const int8_t* gptr, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
+// 16 bytes per lane from global memory (base + offset: a wave-uniform pointer in scalar registers and the lane's
+// 32-bit byte offset) into LDS at lds_addr + 16 * lane (lds_addr is wave-uniform). The form matters: with a 64-bit
+// address per lane the same transfer occupies the CU's address path three to five times as long (measured next to
+// an MFMA stream: about 50 to 80 cycles per instruction against 16, which is the 64 bytes per cycle of the L1).
+__device__ __forceinline__ void global_to_lds_16(const int8_t* base, uint32_t offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(offset), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
@@ -334,7 +337,10 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     // Rows past M and columns past N are clamped into the matrix (what they produce is never stored).
     const int a_row = lane / 4, a_chunk = (lane % 4) ^ ((lane >> 4) & 3);
     const int b_row = lane / 8, b_chunk = (lane % 8) ^ (2 * ((lane >> 4) & 3));
-    struct Cursor { int tile, kt; const int8_t* a[2]; const int8_t* b[2]; } cur;
+    // (a tile's operands as a wave-uniform pointer to its first element plus 32-bit offsets: 127 K + 48 and
+    // 63 N + 112 at most, launch preconditions keep them below 2^31)
+    const int64_t b_step = (int64_t)BK * p.N;
+    struct Cursor { int tile, kt; const int8_t* a_base; const int8_t* b_base; uint32_t a[2], b[2]; } cur;
     auto set_tile = [&](int i) __attribute__((always_inline)) {
         int64_t m0, n0;
         tile_origin(i, m0, n0);
@@ -344,26 +350,27 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
         for (int j = 0; j < 2; ++j) {
             int64_t am = m0 + 16 * (2 * wave + j) + a_row;
             am = am < p.M ? am : p.M - 1;
-            cur.a[j] = p.A + am * p.K + 16 * a_chunk;
-            cur.b[j] = p.B + (int64_t)(8 * (2 * wave + j) + b_row) * p.N + bn;
+            cur.a[j] = (uint32_t)((am - m0) * p.K) + 16u * (uint32_t)a_chunk;
+            cur.b[j] = (uint32_t)(8 * (2 * wave + j) + b_row) * (uint32_t)p.N + (uint32_t)(bn - n0);
         }
+        cur.a_base = p.A + m0 * p.K;
+        cur.b_base = p.B + n0;
         cur.tile = i;
         cur.kt = 0;
     };
-    const int64_t b_step = (int64_t)BK * p.N;
     const uint32_t lds_base = lds_address(lds);
     set_tile(0);
     auto issue_loads = [&](int stage) __attribute__((always_inline)) {
         const uint32_t sa = lds_base + stage * STAGE + 1024 * (2 * wave), sb = sa + A_STAGE;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            global_to_lds_16(cur.a[j], sa + 1024 * j);
-            global_to_lds_16(cur.b[j], sb + 1024 * j);
+            global_to_lds_16(cur.a_base, cur.a[j], sa + 1024 * j);
+            global_to_lds_16(cur.b_base, cur.b[j], sb + 1024 * j);
         }
         if (cur.kt + 1 < ktiles) {
             ++cur.kt;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) { cur.a[j] += BK; cur.b[j] += b_step; }
+            cur.a_base += BK;
+            cur.b_base += b_step;
         } else if (cur.tile + 1 < my_tiles) {
             set_tile(cur.tile + 1);
         }
@@ -635,10 +642,11 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
     p.group_m = 1;
     MI355X_TRACE_INIT(p);
     const Tuning& tune = tuning();
+
     const int cus = device_cus();
     // 16-byte transfers of A rows and B rows; a tile's 128 rows of Y are addressed with 31-bit byte offsets
     if (K > 0 && K % MMF_BK == 0 && N % 16 == 0 && al(A, 16) && al(B, 16) && al(Y, 4) && N < ((int64_t)1 << 21) &&
-        !tune.mmi_generic) {
+        K < ((int64_t)1 << 24) && !tune.mmi_generic) {
         if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "matmul_integer: no usable HIP device");
         // persistent grid: three workgroups per CU (a multiple of the XCD count), fewer if there are fewer tiles
         int64_t grid = (int64_t)(tune.mmi_wgs_per_cu > 0 ? tune.mmi_wgs_per_cu : 3) * (cus / NUM_XCD) * NUM_XCD;

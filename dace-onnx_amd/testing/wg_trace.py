@@ -88,6 +88,8 @@ def trace(name: str, warm_launches: int = 500, max_workgroups: int = 65536):
     d = buf.cpu().numpy().reshape(-1, WORDS)
     d = d[d[:, 0] != 0]
     t = (d[:, :4] - d[:, 0].min()).astype(np.float64) / 100.0
+    extra = np.where(d[:, 5:8] != 0, d[:, 5:8] - d[:, 0].min(), -100).astype(np.float64) / 100.0   # kernel-specific stamps
+    trace.extra = extra
     hw, xcc = d[:, 4] & 0xffffffff, d[:, 4] >> 32
     key = (xcc & 0xf) * 1000 + ((hw >> 13) & 7) * 100 + ((hw >> 12) & 1) * 20 + ((hw >> 8) & 0xf)
     del keep
@@ -105,9 +107,9 @@ def report(name: str):
     print(f"  last workgroup ends at              {t[:, 3].max():.2f}")
     by_cu = {}
     for i in range(len(t)):
-        by_cu.setdefault(int(key[i]), []).append((round(float(t[i, 0]), 2), round(float(t[i, 1]), 2), round(float(t[i, 2]), 2), i))
+        by_cu.setdefault(int(key[i]), []).append(tuple(round(float(v), 2) for v in t[i]) + (i,) + tuple(round(float(v), 2) for v in trace.extra[i]))
     first = sorted(by_cu[int(key[0])])
-    print(f"  the CU of workgroup 0 ran (start, loop entered, loop left, workgroup): {first}")
+    print(f"  the CU of workgroup 0 ran (start, loop entered, loop left, end, workgroup): {first}")
 
 
 if __name__ == "__main__":
