@@ -83,9 +83,17 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     // k = 32*kt + 16*(c*KSPLIT + ks) + 4*lq for its chunks c
     int64_t am = m0 + 16 * wm + li;
     am = am < p.M ? am : p.M - 1;
-    const float* __restrict__ a_ptr = p.A + b0 * p.a_sb0 + b1 * p.a_sb1 + am * p.a_sm + 16 * ks + 4 * lq;
+    // Operands are read as raw buffers: the batch's matrix as the (scalar) base, the lane's row and column as a
+    // 32-bit byte offset, the k-tile as the scalar offset. Next to a stream of MFMAs a load with a 64-bit address
+    // per lane holds up the address path for about 12 cycles, one of this form for 3 or fewer, and the offset
+    // arithmetic per tile leaves the vector unit (launch precondition: a matrix spans less than 2^31 bytes).
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.A + b0 * p.a_sb0 + b1 * p.a_sb1), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.B + b0 * p.b_sb0 + b1 * p.b_sb1), 0, 0x7fffffff, 0x00020000);
+    const uint32_t a_off = (uint32_t)(am * p.a_sm + 16 * ks + 4 * lq) * 4u;
     // this thread's slice of the B tile: row n (clamped), vector c4 of the 32-k row
-    const float* b_ptr[B_PER_T];
+    uint32_t b_off[B_PER_T];
     int b_lds[B_PER_T];
 #pragma unroll
     for (int it = 0; it < B_PER_T; ++it) {
@@ -93,7 +101,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         const int row = idx / (BK / 4), c4 = idx % (BK / 4);
         int64_t bn = n0 + row;
         bn = bn < p.N ? bn : p.N - 1;
-        b_ptr[it] = p.B + b0 * p.b_sb0 + b1 * p.b_sb1 + bn * p.b_sn + 4 * c4;
+        b_off[it] = (uint32_t)(bn * p.b_sn + 4 * c4) * 4u;
         b_lds[it] = row * NT_PITCH + 4 * c4;
     }
 
@@ -108,14 +116,16 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     f32x4 bf[2][TN];           // B fragments of the wave's g-th chunk in set g % 2 (g counts across tiles)
 
     auto load_a = [&](f32x4 (&dst)[NC], int kt) {
+        const int k_bytes = (kt < last_tile ? kt : last_tile) * (BK * 4);
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-            dst[c] = *reinterpret_cast<const f32x4*>(a_ptr + (int64_t)(kt < last_tile ? kt : last_tile) * BK + 16 * c * KSPLIT);
+            dst[c] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_off + 64u * (uint32_t)(c * KSPLIT)), k_bytes, 0));
     };
     auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt) {
+        const int k_bytes = (kt < last_tile ? kt : last_tile) * (BK * 4);
 #pragma unroll
         for (int it = 0; it < B_PER_T; ++it)
-            dst[it] = *reinterpret_cast<const f32x4*>(b_ptr[it] + (int64_t)(kt < last_tile ? kt : last_tile) * BK);
+            dst[it] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, (int)b_off[it], k_bytes, 0));
     };
     auto store_b = [&](const f32x4 (&src)[B_PER_T], int stage) {
         // every thread stores (rows >= BN are padding): no branch in the step body
@@ -266,6 +276,8 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
 // and N a multiple of 4. Additionally needed here: K a multiple of the 32-k tile.
 bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.K % NT_BK != 0 || p.K == 0) return false;
+    // rows are addressed with 32-bit byte offsets from the start of a batch's matrix
+    if ((p.M - 1) * p.a_sm + p.K >= ((int64_t)1 << 29) || (p.N - 1) * p.b_sn + p.K >= ((int64_t)1 << 29)) return false;
     // Candidates: 64x48, 64x64 and 64x144 tiles with two k-split groups, 128x96 tiles without.
     // Cost ~ rounds of workgroups over the CUs x tile area, the large tile discounted
     // for needing half the L2 traffic per FLOP and no reduction.
