@@ -300,7 +300,10 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     // W operand of this lane: row oc (clamped), 4 floats at k = 32 kt + 16 ks + 4 lq
     int64_t am = m0 + 16 * wm + li;
     am = am < p.M ? am : p.M - 1;
-    const float* __restrict__ a_ptr = p.W + am * p.K + 16 * ks + 4 * lq;
+    // (as a raw buffer: the lane's row and k-quad as a 32-bit byte offset, the k-tile as the scalar offset; W spans
+    // less than 2^31 bytes: launch precondition)
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.W), 0, 0x7fffffff, 0x00020000);
+    const uint32_t a_off = (uint32_t)(am * p.K + 16 * ks + 4 * lq) * 4u;
 
     // loader: this thread's output position (the same for all its units): byte offset of
     // its top-left input pixel, and one bit per filter tap (r, s) saying whether that tap
@@ -371,7 +374,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     f32x4 bf[2][TN];           // X operands of tile t in set t % 2
 
     auto load_a = [&](f32x4& dst, int kt) __attribute__((always_inline)) {
-        dst = *reinterpret_cast<const f32x4*>(a_ptr + (int64_t)(kt < last_tile ? kt : last_tile) * BK);
+        dst = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)a_off, (kt < last_tile ? kt : last_tile) * (BK * 4), 0));
     };
     auto load_b = [&](f32x4 (&dst)[B_PER_T], int kt, auto i_tag) __attribute__((always_inline)) {
         constexpr int I = decltype(i_tag)::value;   // the step's place in its window (compile-time taps)
@@ -646,7 +649,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
     hipStream_t st = static_cast<hipStream_t>(stream);
     p.group_m = 1;
     // K a multiple of the 32-k tile and 16-byte aligned W rows: the gather kernel
-    if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && C * H * Wd < ((int64_t)1 << 27) &&
+    if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && M * K < ((int64_t)1 << 29) && C * H * Wd < ((int64_t)1 << 27) &&
         N * C * H * Wd + pads[0] * Wd + pads[1] + H * Wd < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
         p.x_bytes = (int)(N * C * H * Wd * 4);
         // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
