@@ -42,7 +42,7 @@ int device_cus();
 #define MI355X_TRACE_INIT(args) (args).trace = ::mi355x::trace_buffer()
 #define MI355X_TRACE_STAMP(args, slot)                                                          \
     do {                                                                                        \
-        if ((args).trace && threadIdx.x == 0) (args).trace[8 * blockIdx.x + (slot)] = wall_clock64(); \
+        if ((args).trace && threadIdx.x == 0) (args).trace[16 * blockIdx.x + (slot)] = wall_clock64(); \
     } while (0)
 #define MI355X_TRACE_HWID(args)                                                                 \
     do {                                                                                        \
@@ -50,7 +50,7 @@ int device_cus();
             unsigned hw_, xcc_;                                                                 \
             asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_));                   \
             asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_));                 \
-            (args).trace[8 * blockIdx.x + 4] = ((unsigned long long)xcc_ << 32) | hw_;          \
+            (args).trace[16 * blockIdx.x + 4] = ((unsigned long long)xcc_ << 32) | hw_;          \
         }                                                                                       \
     } while (0)
 unsigned long long* trace_buffer();

@@ -506,15 +506,21 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
             for (int j = 0; j < TN; ++j) red[(wm * TN + j) * WAVE + lane] = acc[j];
         }
         __syncthreads();
+        MI355X_TRACE_STAMP(p, 8);
         if (ks == 1) return;
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[j] += red[(wm * TN + j) * WAVE + lane];
     }
+    MI355X_TRACE_STAMP(p, 9);
 
     // epilogue: acc[j][r] = Y[oc = m0 + 16 wm + li][p = p0 + 16 j + 4 lq + r]
     const int64_t oc = m0 + 16 * wm + li;
     if (oc >= p.M) return;
     const float bv = (p.epi & MI355X_EPI_BIAS) ? p.bias[oc] : 0.f;
+#ifdef MI355X_WG_TRACE
+    asm volatile("" :: "v"(bv));
+    MI355X_TRACE_STAMP(p, 10);
+#endif
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int64_t pp = p0 + 16 * j + 4 * lq;

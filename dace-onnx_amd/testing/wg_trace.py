@@ -12,7 +12,10 @@ What the stamps mean per kernel (microseconds; the wall clock ticks at 100 MHz):
 * slot 0 start, slot 1 main loop entered (first operands arrived), slot 2 main loop left (by the first wave),
   slot 3 last store issued -- for MatMulInteger: last store acknowledged;
 * workgroups are grouped by CU through the hardware id register to show which of them share a CU and when each of
-  them was in its loop.
+  them was in its loop;
+* the convolution adds six more, printed after the workgroup's number in the per-CU list: set-up done (first
+  barrier), first six steps' loads issued, their first two stored to LDS; after the loop: partial sums of the
+  second k-split group exchanged, added, bias arrived (-1 where a kernel has no such stamp).
 """
 import ctypes
 import os
@@ -23,7 +26,7 @@ import numpy as np
 from .. import _lib
 
 TRACE_LIBRARY = os.path.join(os.path.dirname(_lib.LIBRARY_PATH), "libmi355x_onnx_trace.so")
-WORDS = 8   # 64-bit words per workgroup in the trace buffer
+WORDS = 16   # 64-bit words per workgroup in the trace buffer
 
 
 def load_trace_library():
@@ -88,7 +91,7 @@ def trace(name: str, warm_launches: int = 500, max_workgroups: int = 65536):
     d = buf.cpu().numpy().reshape(-1, WORDS)
     d = d[d[:, 0] != 0]
     t = (d[:, :4] - d[:, 0].min()).astype(np.float64) / 100.0
-    extra = np.where(d[:, 5:8] != 0, d[:, 5:8] - d[:, 0].min(), -100).astype(np.float64) / 100.0   # kernel-specific stamps
+    extra = np.where(d[:, 5:11] != 0, d[:, 5:11] - d[:, 0].min(), -100).astype(np.float64) / 100.0   # kernel-specific stamps
     trace.extra = extra
     hw, xcc = d[:, 4] & 0xffffffff, d[:, 4] >> 32
     key = (xcc & 0xf) * 1000 + ((hw >> 13) & 7) * 100 + ((hw >> 12) & 1) * 20 + ((hw >> 8) & 0xf)
