@@ -194,11 +194,13 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         __syncthreads();
     };
 
+    MI355X_TRACE_STAMP(p, 5);
 #pragma unroll
     for (int r = 0; r < RING; ++r) {  // tiles beyond the last are clamped: no branch
         load_a(ra[r], r);
         load_b(rb[r], r);
     }
+    MI355X_TRACE_STAMP(p, 6);
     // The small-tile variants have registers to spare: fetch this lane's bias and residual
     // values now, so the epilogue does not wait for two more trips to memory (k-split
     // group 1 never needs them).
@@ -218,6 +220,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     }
     store_b(rb[0], 0);
     store_b(rb[1], 1);
+    MI355X_TRACE_STAMP(p, 7);
     __syncthreads();
     read_b(bf[0], 0, 0);
     MI355X_TRACE_STAMP(p, 1);
