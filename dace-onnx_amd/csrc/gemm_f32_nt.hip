@@ -280,7 +280,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
 bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.K % NT_BK != 0 || p.K == 0) return false;
     // rows are addressed with 32-bit byte offsets from the start of a batch's matrix
-    if ((p.M - 1) * p.a_sm + p.K >= ((int64_t)1 << 29) || (p.N - 1) * p.b_sn + p.K >= ((int64_t)1 << 29)) return false;
+    if (p.a_sm < 0 || p.b_sn < 0 || (p.M - 1) * p.a_sm + p.K >= ((int64_t)1 << 29) || (p.N - 1) * p.b_sn + p.K >= ((int64_t)1 << 29)) return false;
     // Candidates: 64x48, 64x64 and 64x144 tiles with two k-split groups, 128x96 tiles without.
     // Cost ~ rounds of workgroups over the CUs x tile area, the large tile discounted
     // for needing half the L2 traffic per FLOP and no reduction.
