@@ -35,8 +35,8 @@ int device_cus();
 // Workgroup trace, compiled in only with -DMI355X_WG_TRACE (`make trace` builds libmi355x_onnx_trace.so): the contraction
 // kernels stamp the wall clock (100 MHz) at the start of a workgroup, at the first and after the last step of its main
 // loop and at its end, plus the hardware id of the CU it runs on, into the buffer whose device address the environment
-// variable MI355X_WG_TRACE_BUFFER holds (8 x 64-bit words per workgroup; unset: no stamps). The normal build carries
-// neither the argument nor the code.
+// variable MI355X_WG_TRACE_BUFFER holds (16 x 64-bit words per workgroup: slots 0-3 the four stamps, 4 the hardware id,
+// 5 and up kernel-specific stamps; unset: no stamps). The normal build carries neither the argument nor the code.
 #ifdef MI355X_WG_TRACE
 #define MI355X_TRACE_MEMBER unsigned long long* trace;
 #define MI355X_TRACE_INIT(args) (args).trace = ::mi355x::trace_buffer()
