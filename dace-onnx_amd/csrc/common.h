@@ -36,13 +36,17 @@ int device_cus();
 // kernels stamp the wall clock (100 MHz) at the start of a workgroup, at the first and after the last step of its main
 // loop and at its end, plus the hardware id of the CU it runs on, into the buffer whose device address the environment
 // variable MI355X_WG_TRACE_BUFFER holds (16 x 64-bit words per workgroup: slots 0-3 the four stamps, 4 the hardware id,
-// 5 and up kernel-specific stamps; unset: no stamps). The normal build carries neither the argument nor the code.
+// 5 to 11 kernel-specific stamps, 12 and 13 the shader cycle counter at the loop's first and after its last step; unset: no stamps). The normal build carries neither the argument nor the code.
 #ifdef MI355X_WG_TRACE
 #define MI355X_TRACE_MEMBER unsigned long long* trace;
 #define MI355X_TRACE_INIT(args) (args).trace = ::mi355x::trace_buffer()
 #define MI355X_TRACE_STAMP(args, slot)                                                          \
     do {                                                                                        \
         if ((args).trace && threadIdx.x == 0) (args).trace[16 * blockIdx.x + (slot)] = wall_clock64(); \
+    } while (0)
+#define MI355X_TRACE_CYCLES(args, slot)                                                         \
+    do {                                                                                        \
+        if ((args).trace && threadIdx.x == 0) (args).trace[16 * blockIdx.x + (slot)] = __builtin_readcyclecounter(); \
     } while (0)
 #define MI355X_TRACE_HWID(args)                                                                 \
     do {                                                                                        \
@@ -58,6 +62,7 @@ unsigned long long* trace_buffer();
 #define MI355X_TRACE_MEMBER
 #define MI355X_TRACE_INIT(args) do {} while (0)
 #define MI355X_TRACE_STAMP(args, slot) do {} while (0)
+#define MI355X_TRACE_CYCLES(args, slot) do {} while (0)
 #define MI355X_TRACE_HWID(args) do {} while (0)
 #endif
 

@@ -488,6 +488,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     // compiler's wait-count analysis drains every outstanding load at the loop header); the at most
     // RING - 1 remaining steps follow, guarded.
     MI355X_TRACE_STAMP(p, 1);
+    MI355X_TRACE_CYCLES(p, 12);
     int kt0 = 0;
     for (; kt0 + UNROLL <= ktiles; kt0 += UNROLL) {
         cg_static_for<UNROLL>([&](auto u_tag) __attribute__((always_inline)) { tile_step(u_tag, kt0 + decltype(u_tag)::value); });
@@ -498,6 +499,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     });
 
     MI355X_TRACE_STAMP(p, 2);
+    MI355X_TRACE_CYCLES(p, 13);
     // k-split group 1 hands its partial sums to group 0 through LDS
     {
         f32x4* red = reinterpret_cast<f32x4*>(lds);

@@ -224,6 +224,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     __syncthreads();
     read_b(bf[0], 0, 0);
     MI355X_TRACE_STAMP(p, 1);
+    MI355X_TRACE_CYCLES(p, 12);
 
     // One code path for every tile: near the end of K the look-aheads are not switched
     // off but clamped to the last tile (they re-read data that is already in cache and
@@ -238,6 +239,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     }
 
     MI355X_TRACE_STAMP(p, 2);
+    MI355X_TRACE_CYCLES(p, 13);
     // k-split group 1 hands its partial sums to group 0 through LDS
     if constexpr (KSPLIT == 2) {
         f32x4* red = reinterpret_cast<f32x4*>(lds);

@@ -561,6 +561,7 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     }
     __syncthreads();
     MI355X_TRACE_STAMP(p, 1);   // the first operands are in LDS
+    MI355X_TRACE_CYCLES(p, 12);
     read_frags(0, 0, 0);
 
     int kt = 0, tile_i = 0, stage = 0;
@@ -593,6 +594,7 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
         stage = stage1;
     }
     MI355X_TRACE_STAMP(p, 2);
+    MI355X_TRACE_CYCLES(p, 13);
     if (pending) finish_tile(tile_i - 1);
 #ifdef MI355X_WG_TRACE
     if (p.trace) MI355X_WAIT_VMCNT(0);   // slot 3: the last store is acknowledged
