@@ -4,6 +4,7 @@ reference's, refusals are reported, and the ONNX reader/shape inference work."""
 import ctypes
 import os
 import re
+import subprocess
 
 import numpy as np
 import pytest
@@ -413,3 +414,16 @@ def test_onnx_model_helpers_of_the_reference_api():
     assert tuple(out.shape) == tuple(desc.shape) and out.dtype == torch.float32 and float(out.abs().sum()) == 0.0
     with pytest.raises(ValueError, match="use_torch=False"):
         create_output_array({}, desc, use_torch=False)
+
+
+def test_trace_build_is_separate_from_the_library(monkeypatch, tmp_path):
+    """The workgroup trace lives in a second build (`make trace`): the script that reads it asks for that file by name and
+    says how to build it when it is missing; the product library exports no trace symbol."""
+    from dace_onnx_amd.testing import wg_trace
+    assert os.path.basename(wg_trace.TRACE_LIBRARY) == "libmi355x_onnx_trace.so"
+    assert os.path.dirname(wg_trace.TRACE_LIBRARY) == os.path.dirname(_lib.LIBRARY_PATH)
+    monkeypatch.setattr(wg_trace, "TRACE_LIBRARY", str(tmp_path / "absent.so"))
+    with pytest.raises(_lib.LibraryNotBuilt, match="make -C dace-onnx_amd/csrc trace"):
+        wg_trace.load_trace_library()
+    exported = subprocess.run(["nm", "-D", "--defined-only", _lib.LIBRARY_PATH], capture_output=True, text=True, check=True).stdout
+    assert "trace_buffer" not in exported
