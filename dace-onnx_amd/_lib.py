@@ -39,6 +39,7 @@ SIGNATURES: typing.Dict[str, typing.Tuple[typing.Any, typing.List[typing.Any]]] 
     "mi355x_last_error": (ctypes.c_char_p, []),
     "mi355x_device_cu_count": (_int, []),
     "mi355x_reload_tuning": (None, []),
+    "mi355x_launch_empty_kernel": (_int, [_vp]),
     "mi355x_gemm_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                _c_i64_p, _c_i64_p, _c_i64_p, _c_i64_p, _f32, _int, _vp]),
     "mi355x_conv2d_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,

@@ -34,9 +34,11 @@ static std::atomic<bool> g_tuning_valid{false};
 static std::mutex g_tuning_mutex;
 
 #ifdef MI355X_WG_TRACE
-unsigned long long* trace_buffer() {
+unsigned long long* trace_buffer(unsigned* capacity) {
     const char* v = getenv("MI355X_WG_TRACE_BUFFER");
-    return v && *v ? reinterpret_cast<unsigned long long*>(strtoull(v, nullptr, 10)) : nullptr;
+    const char* c = getenv("MI355X_WG_TRACE_CAPACITY");
+    *capacity = c && *c ? (unsigned)strtoul(c, nullptr, 10) : 0u;
+    return v && *v && *capacity ? reinterpret_cast<unsigned long long*>(strtoull(v, nullptr, 10)) : nullptr;
 }
 #endif
 
@@ -60,13 +62,12 @@ static void parse_tuning(Tuning& t) {
     t.mmi_wgs_per_cu = env_int("MI355X_MMI_WGS_PER_CU", 0);
 }
 
-const Tuning& tuning() {
-    if (!g_tuning_valid.load(std::memory_order_acquire)) {
-        std::lock_guard<std::mutex> lock(g_tuning_mutex);
-        if (!g_tuning_valid.load(std::memory_order_relaxed)) {
-            parse_tuning(g_tuning);
-            g_tuning_valid.store(true, std::memory_order_release);
-        }
+Tuning tuning() {
+    // every read of the struct happens under the lock mi355x_reload_tuning() writes it under; a launch works on its copy
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);
+    if (!g_tuning_valid.load(std::memory_order_relaxed)) {
+        parse_tuning(g_tuning);
+        g_tuning_valid.store(true, std::memory_order_relaxed);
     }
     return g_tuning;
 }
@@ -88,9 +89,16 @@ int device_cus() {
     return cus;
 }
 
+__global__ void empty_kernel() {}
+
 }  // namespace mi355x
 
 extern "C" {
+
+int mi355x_launch_empty_kernel(void* stream) {
+    hipLaunchKernelGGL(mi355x::empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream));
+    return mi355x::check_launch("empty_kernel");
+}
 
 void mi355x_reload_tuning(void) {
     std::lock_guard<std::mutex> lock(mi355x::g_tuning_mutex);

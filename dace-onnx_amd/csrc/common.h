@@ -29,35 +29,38 @@ struct Tuning {
     bool mmi_generic = false;
     int mmi_wgs_per_cu = 0;
 };
-const Tuning& tuning();
+Tuning tuning();   // a copy taken under the lock: a reload never changes what a launch in progress reads
 int device_cus();
 
 // Workgroup trace, compiled in only with -DMI355X_WG_TRACE (`make trace` builds libmi355x_onnx_trace.so): the contraction
 // kernels stamp the wall clock (100 MHz) at the start of a workgroup, at the first and after the last step of its main
 // loop and at its end, plus the hardware id of the CU it runs on, into the buffer whose device address the environment
 // variable MI355X_WG_TRACE_BUFFER holds (16 x 64-bit words per workgroup: slots 0-3 the four stamps, 4 the hardware id,
-// 5 to 11 kernel-specific stamps, 12 and 13 the shader cycle counter at the loop's first and after its last step; unset: no stamps). The normal build carries neither the argument nor the code.
+// 5 to 11 kernel-specific stamps, 12 and 13 the shader cycle counter at the loop's first and after its last step; unset: no
+// stamps). MI355X_WG_TRACE_CAPACITY holds the number of workgroups the buffer has room for: workgroups beyond it write
+// nothing, and without it no stamp is written at all. The normal build carries neither the arguments nor the code.
 #ifdef MI355X_WG_TRACE
-#define MI355X_TRACE_MEMBER unsigned long long* trace;
-#define MI355X_TRACE_INIT(args) (args).trace = ::mi355x::trace_buffer()
+#define MI355X_TRACE_MEMBER unsigned long long* trace; unsigned trace_capacity;
+#define MI355X_TRACE_INIT(args) (args).trace = ::mi355x::trace_buffer(&(args).trace_capacity)
+#define MI355X_TRACE_ON(args) ((args).trace && threadIdx.x == 0 && blockIdx.x < (args).trace_capacity)
 #define MI355X_TRACE_STAMP(args, slot)                                                          \
     do {                                                                                        \
-        if ((args).trace && threadIdx.x == 0) (args).trace[16 * blockIdx.x + (slot)] = wall_clock64(); \
+        if (MI355X_TRACE_ON(args)) (args).trace[16 * blockIdx.x + (slot)] = wall_clock64(); \
     } while (0)
 #define MI355X_TRACE_CYCLES(args, slot)                                                         \
     do {                                                                                        \
-        if ((args).trace && threadIdx.x == 0) (args).trace[16 * blockIdx.x + (slot)] = __builtin_readcyclecounter(); \
+        if (MI355X_TRACE_ON(args)) (args).trace[16 * blockIdx.x + (slot)] = __builtin_readcyclecounter(); \
     } while (0)
 #define MI355X_TRACE_HWID(args)                                                                 \
     do {                                                                                        \
-        if ((args).trace && threadIdx.x == 0) {                                                 \
+        if (MI355X_TRACE_ON(args)) {                                                 \
             unsigned hw_, xcc_;                                                                 \
             asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_));                   \
             asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_));                 \
             (args).trace[16 * blockIdx.x + 4] = ((unsigned long long)xcc_ << 32) | hw_;          \
         }                                                                                       \
     } while (0)
-unsigned long long* trace_buffer();
+unsigned long long* trace_buffer(unsigned* capacity);
 #else
 #define MI355X_TRACE_MEMBER
 #define MI355X_TRACE_INIT(args) do {} while (0)

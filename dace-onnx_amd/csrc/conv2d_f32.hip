@@ -580,8 +580,7 @@ struct ConvTile { int bm, bn; };
 static const ConvTile kConvTiles[] = {{64, 128}, {64, 64}, {32, 64}, {16, 64}, {128, 64}};
 constexpr int kNumConvTiles = sizeof(kConvTiles) / sizeof(kConvTiles[0]);
 
-static int choose_conv_tile(int64_t M, int64_t P, int cus) {
-    const int force = tuning().conv_config;
+static int choose_conv_tile(int64_t M, int64_t P, int cus, int force) {
     if (force >= 0 && force < kNumConvTiles) return force;
     double best = 1e300;
     int best_cfg = 1;
@@ -654,11 +653,12 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
 
     const int cus = device_cus();
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "conv2d: no usable HIP device");
+    const Tuning tune = tuning();
     hipStream_t st = static_cast<hipStream_t>(stream);
     p.group_m = 1;
     // K a multiple of the 32-k tile and 16-byte aligned W rows: the gather kernel
     if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && M * K < ((int64_t)1 << 29) && C * H * Wd < ((int64_t)1 << 27) &&
-        N * C * H * Wd + pads[0] * Wd + pads[1] + H * Wd < ((int64_t)1 << 29) && al16(W) && tuning().conv_config < 0) {
+        N * C * H * Wd + pads[0] * Wd + pads[1] + H * Wd < ((int64_t)1 << 29) && al16(W) && tune.conv_config < 0) {
         p.x_bytes = (int)(N * C * H * Wd * 4);
         // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
         // at the same rate, so the choice is the number of rounds times the tile width; ties go
@@ -667,7 +667,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
             const int64_t tiles = ceil_div(M, (int64_t)CG_BM) * ceil_div(P, (int64_t)bn);
             return ceil_div(tiles, (int64_t)cus * wgs_per_cu) * bn * wgs_per_cu;
         };
-        const bool wide = tuning().conv_gather_bn ? tuning().conv_gather_bn == 128 : cost(128, 1) < cost(64, 2);
+        const bool wide = tune.conv_gather_bn ? tune.conv_gather_bn == 128 : cost(128, 1) < cost(64, 2);
         const int bn = wide ? 128 : 64;
         p.tiles_m = ceil_div(M, (int64_t)CG_BM);
         p.tiles_p = ceil_div(P, (int64_t)bn);
@@ -678,10 +678,10 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
         // 1568 tiles on 512 places): the tiles of that round run as 16-position slices, four times as many
         // workgroups of a quarter of the work each, so the places that would idle through a whole tile time
         // share its work.
-        if (!wide && tuning().conv_tail != 0) {
+        if (!wide && tune.conv_tail != 0) {
             const int64_t places = (int64_t)cus * 2, rem = p.full_tiles % places;
-            const int64_t tail_p = tuning().conv_tail > 0 ? tuning().conv_tail : rem / p.tiles_m;
-            const bool wanted = tuning().conv_tail > 0 || (p.full_tiles > places && rem > 0 && rem < places / 2);
+            const int64_t tail_p = tune.conv_tail > 0 ? tune.conv_tail : rem / p.tiles_m;
+            const bool wanted = tune.conv_tail > 0 || (p.full_tiles > places && rem > 0 && rem < places / 2);
             if (wanted && tail_p > 0 && tail_p < p.tiles_p) {
                 p.tiles_p -= tail_p;
                 p.full_tiles = p.tiles_m * p.tiles_p;
@@ -692,7 +692,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
         p.nwg = p.full_tiles + slices;
         MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "conv2d: grid too large");
         // 3 x 3 and 1 x 1 filters over whole windows of 32 channels: taps known at compile time
-        const int taps = (C % 32 == 0 && (KH * KW == 9 || KH * KW == 1) && tuning().conv_static_taps) ? (int)(KH * KW) : 0;
+        const int taps = (C % 32 == 0 && (KH * KW == 9 || KH * KW == 1) && tune.conv_static_taps) ? (int)(KH * KW) : 0;
         const dim3 g((unsigned)p.nwg), b(CG_THREADS);
         if (wide) {
             if (taps == 9) hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 9>), g, b, 0, st, p);
@@ -705,7 +705,7 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
         }
         return check_launch("conv2d_f32_gather_kernel");
     }
-    const int cfg = choose_conv_tile(M, P, cus);
+    const int cfg = choose_conv_tile(M, P, cus, tune.conv_config);
     p.tiles_m = ceil_div(M, kConvTiles[cfg].bm);
     p.tiles_p = ceil_div(P, kConvTiles[cfg].bn);
     p.nwg = p.tiles_m * p.tiles_p;

@@ -292,7 +292,7 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     const Cand cands[] = {{64, 48, 1.0}, {64, 64, 1.0}, {128, 96, 0.8}, {64, 144, 1.0}};
     int best = 0;
     double best_cost = 1e300;
-    const Tuning& tune = tuning();
+    const Tuning tune = tuning();
     const int force = tune.gemm_nt_bn;
     for (int c = 0; c < 4; ++c) {
         const int64_t nwg = p.batch * ceil_div(p.M, cands[c].bm) * ceil_div(p.N, cands[c].bn);

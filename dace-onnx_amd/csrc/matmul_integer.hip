@@ -294,6 +294,12 @@ __device__ __forceinline__ i32x2 lds_read_tr8(const uint8_t* p) {
 // address per lane the same transfer occupies the CU's address path three to five times as long (measured next to
 // an MFMA stream: about 50 to 80 cycles per instruction against 16, which is the 64 bytes per cycle of the L1).
 __device__ __forceinline__ void global_to_lds_16(const int8_t* base, uint32_t offset, uint32_t lds_addr) {
+    // the pointer is wave-uniform by construction; saying so keeps it in scalar registers whatever the compiler can prove
+    // (a no-op where it already holds it there)
+    const uint64_t b64 = reinterpret_cast<uint64_t>(base);
+    base = reinterpret_cast<const int8_t*>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b64 >> 32)) << 32) |
+                                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64));
+    lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(offset), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
@@ -643,7 +649,7 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
     hipStream_t st = static_cast<hipStream_t>(stream);
     p.group_m = 1;
     MI355X_TRACE_INIT(p);
-    const Tuning& tune = tuning();
+    const Tuning tune = tuning();
 
     const int cus = device_cus();
     // 16-byte transfers of A rows and B rows; a tile's 128 rows of Y are addressed with 31-bit byte offsets

@@ -85,9 +85,13 @@ def trace(name: str, warm_launches: int = 500, max_workgroups: int = 65536):
     torch.cuda.synchronize()
     buf = torch.zeros(WORDS * max_workgroups, dtype=torch.int64, device="cuda")
     os.environ["MI355X_WG_TRACE_BUFFER"] = str(buf.data_ptr())
-    status = launch()
-    torch.cuda.synchronize()
-    os.environ.pop("MI355X_WG_TRACE_BUFFER", None)
+    os.environ["MI355X_WG_TRACE_CAPACITY"] = str(max_workgroups)   # workgroups beyond it write no stamps
+    try:
+        status = launch()
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("MI355X_WG_TRACE_BUFFER", None)
+        os.environ.pop("MI355X_WG_TRACE_CAPACITY", None)
     if status != 0:
         raise _lib.MI355XError(lib.mi355x_last_error().decode())
     d = buf.cpu().numpy().reshape(-1, WORDS)

@@ -52,6 +52,11 @@ const char* mi355x_last_error(void);
  * Used by callers that size grids or report occupancy; no reference counterpart. */
 int mi355x_device_cu_count(void);
 
+/* Launches one workgroup of a kernel that does nothing, on `stream`. What such a launch costs is the floor under every
+ * kernel duration on the part; a benchmark measures it to say how much of a small kernel's time is the launch itself.
+ * No reference counterpart (the reference times whole programs, daceml/testing/profiling/event_profiler.py:87-143). */
+int mi355x_launch_empty_kernel(void* stream);
+
 /* The MI355X_* environment variables that force a kernel variant (MI355X_GEMM_CONFIG, MI355X_GEMM_NT_BN,
  * MI355X_GEMM_NT_BK, MI355X_GEMM_GROUP_M, MI355X_CONV_CONFIG, MI355X_CONV_GATHER_BN, MI355X_CONV_TAIL, MI355X_CONV_STATIC_TAPS, MI355X_MMI_GENERIC,
  * MI355X_MMI_WGS_PER_CU) are read on the first launch only; call this after changing them. The role of

@@ -49,3 +49,34 @@ def rel_err(expected, actual):
 #: fp32 parity bar for every floating-point kernel: 1e-4 relative to the largest
 #: magnitude of the expected tensor (integer kernels must be bit-exact)
 FP32_REL_TOL = 1e-4
+
+
+@pytest.fixture
+def tuning():
+    """Forces kernel variants through the library's ``MI355X_*`` variables: ``tuning(MI355X_GEMM_NT_BN="48")`` sets
+    them (``None`` unsets one) and has the library read them again. Whatever happens in the test, the variables are
+    taken back and the library re-reads its own choice before the next test runs (the library reads them once and
+    caches what it found)."""
+    from dace_onnx_amd import _lib
+    lib = _lib.library()
+    before = {}
+
+    def force(**variables):
+        for name, value in variables.items():
+            assert name.startswith("MI355X_"), name
+            before.setdefault(name, os.environ.get(name))
+            if value is None:
+                os.environ.pop(name, None)
+            else:
+                os.environ[name] = str(value)
+        lib.mi355x_reload_tuning()
+
+    try:
+        yield force
+    finally:
+        for name, value in before.items():
+            if value is None:
+                os.environ.pop(name, None)
+            else:
+                os.environ[name] = value
+        lib.mi355x_reload_tuning()

@@ -273,15 +273,11 @@ def test_strided_gemm_head_split_merge_without_copies():
 @pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144"])
 @pytest.mark.parametrize("M, N, K, epi", [(64, 48, 32, 0), (1, 4, 32, 1), (130, 52, 64, 9), (257, 100, 96, 5), (200, 148, 160, 3),
                                           (1024, 768, 768, 9), (63, 764, 224, 8), (100, 52, 2112, 9)])   # last: 64-k tiles
-def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
+def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
     """Both operands k-contiguous (activations x [N, K] weights): every tile variant of that kernel on shapes that
     leave partial tiles in M and N, with each epilogue combination (1 bias, 2 relu, 4 gelu, 8 residual) and alpha."""
-    if tile == "auto":
-        monkeypatch.delenv("MI355X_GEMM_NT_BN", raising=False)
-    else:
-        monkeypatch.setenv("MI355X_GEMM_NT_BN", tile)
+    tuning(MI355X_GEMM_NT_BN=None if tile == "auto" else tile)   # the variables are read once; the fixture reloads them
     lib = _lib.library()
-    lib.mi355x_reload_tuning()   # the variables are read once; this test changes them between calls
     rng = np.random.default_rng(M * 7 + N * 3 + K + epi)
     a = torch.from_numpy(rng.normal(size=(2, M, K)).astype(np.float32)).cuda()
     w = torch.from_numpy(rng.normal(size=(N, K)).astype(np.float32)).cuda()          # [N, K]: B[k, n] = w[n, k]
@@ -301,9 +297,61 @@ def test_k_contiguous_gemm_tiles_and_epilogues(monkeypatch, tile, M, N, K, epi):
         ref = torch.nn.functional.gelu(ref)
     if epi & 8:
         ref = ref + res.double()
-    monkeypatch.delenv("MI355X_GEMM_NT_BN", raising=False)
-    lib.mi355x_reload_tuning()   # back to the library's own choice for the tests that follow
     assert rel_err(ref.cpu().numpy(), out.cpu().numpy()) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("variables", [{"MI355X_GEMM_CONFIG": c} for c in range(5)] + [{"MI355X_GEMM_NT_BK": 32},
+                                                                                        {"MI355X_GEMM_NT_BK": 32, "MI355X_GEMM_NT_BN": 64},
+                                                                                        {"MI355X_GEMM_GROUP_M": 1}])
+@pytest.mark.parametrize("M, N, K, epi", [(130, 100, 64, 9), (257, 52, 2112, 5)])
+def test_forced_gemm_variants(tuning, variables, M, N, K, epi):
+    """Every tile shape of the generic double-buffered kernel (which the library itself only picks for operands that are
+    not both k-contiguous), the 32-k walk of the k-contiguous kernel where it would pick 64-k tiles, and a forced
+    panel height, on the k-contiguous problem: each must give the float64 product within the fp32 bar."""
+    tuning(**variables)
+    lib = _lib.library()
+    rng = np.random.default_rng(M + N + K)
+    a = torch.from_numpy(rng.normal(size=(M, K)).astype(np.float32)).cuda()
+    w = torch.from_numpy(rng.normal(size=(N, K)).astype(np.float32)).cuda()
+    bias = torch.from_numpy(rng.normal(size=N).astype(np.float32)).cuda()
+    res = torch.from_numpy(rng.normal(size=(M, N)).astype(np.float32)).cuda()
+    out = torch.full((M, N), float("nan"), device="cuda")
+    _lib.check(lib.mi355x_gemm_f32(a.data_ptr(), w.data_ptr(), out.data_ptr(), bias.data_ptr(), res.data_ptr(), 1, 1, M, N, K,
+                                   _lib.i64_array([0, 0, K, 1]), _lib.i64_array([0, 0, 1, K]), _lib.i64_array([0, 0, N]),
+                                   _lib.i64_array([0, 0, N]), 1.0, epi, _lib.current_stream()), "gemm")
+    ref = a.double() @ w.double().T + bias.double()
+    if epi & 4:
+        ref = torch.nn.functional.gelu(ref)
+    if epi & 8:
+        ref = ref + res.double()
+    assert rel_err(ref.cpu().numpy(), out.cpu().numpy()) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("config", range(5))
+def test_forced_conv_tile_variants(tuning, config):
+    """MI355X_CONV_CONFIG sends a convolution the gather kernel would take to each tile shape of the generic kernel."""
+    tuning(MI355X_CONV_CONFIG=config)
+    rng = np.random.default_rng(40 + config)
+    x = rng.normal(size=(2, 32, 13, 11)).astype(np.float32)
+    w = (rng.normal(size=(40, 32, 3, 3)) / 17.0).astype(np.float32)
+    b = rng.normal(size=40).astype(np.float32)
+    y = np.zeros((2, 40, 13, 11), np.float32)
+    donnx.ONNXConv(X=x, W=w, B=b, Y=y, pads=[1, 1, 1, 1])
+    assert rel_err(O.conv2d(x, w, b, pads=(1, 1, 1, 1)), y) < FP32_REL_TOL
+
+
+@pytest.mark.parametrize("variables", [{"MI355X_MMI_GENERIC": 1}, {"MI355X_MMI_WGS_PER_CU": 1}, {"MI355X_MMI_WGS_PER_CU": 2}])
+def test_forced_matmul_integer_variants(tuning, variables):
+    """The generic MatMulInteger kernel on a shape the streaming kernel would take, and the streaming kernel with fewer
+    workgroups per CU than it picks: bit-exact against the int64 formula."""
+    tuning(**variables)
+    rng = np.random.default_rng(55)
+    A = rng.integers(-128, 128, size=(384, 192), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(192, 272), dtype=np.int8)
+    Y = np.zeros((384, 272), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array(3, np.int8), b_zero_point=np.array(-2, np.int8), Y=Y)
+    want = (A.astype(np.int64) - 3) @ (B.astype(np.int64) + 2)
+    assert np.array_equal(want, Y)
 
 
 def test_save_transients_keeps_every_intermediate(golden):
@@ -500,7 +548,7 @@ def test_conv_residual_epilogue(shape, wshape, pads, strides, epi):
     ((2, 64, 16, 16), (80, 64, 3, 3), 7),      # two tiles of output channels (the second partly filled), 1 whole tile per row of tiles
     ((1, 32, 9, 9), (16, 32, 3, 3), 1)])       # 81 positions, odd: scalar stores in the slices
 @pytest.mark.parametrize("epi", [0, _lib.EPI_BIAS | _lib.EPI_RELU, _lib.EPI_BIAS | _lib.EPI_RESIDUAL | _lib.EPI_RELU_AFTER])
-def test_conv_last_round_as_slices(monkeypatch, shape, wshape, tail, epi):
+def test_conv_last_round_as_slices(tuning, shape, wshape, tail, epi):
     """The convolution's last round of tiles run as 16-position slices (the library chooses that by the number of
     tiles and CUs; here it is forced on small problems through MI355X_CONV_TAIL = number of position tiles to slice)."""
     rng = np.random.default_rng(31 + tail)
@@ -520,14 +568,11 @@ def test_conv_last_round_as_slices(monkeypatch, shape, wshape, tail, epi):
                       torch.cuda.current_stream().cuda_stream]
     results = []
     for setting in (str(tail), "0"):
-        monkeypatch.setenv("MI355X_CONV_TAIL", setting)
-        lib.mi355x_reload_tuning()
+        tuning(MI355X_CONV_TAIL=setting)
         y = torch.full(pre.shape, float("nan"), device="cuda")
         assert lib.mi355x_conv2d_res_f32(*args(y)) == 0, lib.mi355x_last_error()
         torch.cuda.synchronize()
         results.append(y.cpu().numpy())
-    monkeypatch.delenv("MI355X_CONV_TAIL", raising=False)
-    lib.mi355x_reload_tuning()
     assert rel_err(expected, results[0]) < FP32_REL_TOL
     # a slice adds up the same products in the same order as the tile it stands in for
     assert np.array_equal(results[0], results[1])
@@ -541,7 +586,7 @@ def test_conv_last_round_as_slices(monkeypatch, shape, wshape, tail, epi):
     ((1, 32, 10, 7), (16, 32, 1, 9), (1, 1), (0, 4, 0, 4), (1, 1), 64),      # nine taps in one row
     ((3, 64, 9, 9), (64, 64, 1, 1), (1, 1), (0, 0, 0, 0), (1, 1), 64),       # 1 x 1
     ((2, 224, 8, 8), (40, 224, 1, 1), (2, 2), (0, 0, 0, 0), (1, 1), 128)])   # 1 x 1, stride 2, 7 steps
-def test_conv_taps_known_at_compile_time(monkeypatch, shape, wshape, strides, pads, dilations, gather_bn):
+def test_conv_taps_known_at_compile_time(tuning, shape, wshape, strides, pads, dilations, gather_bn):
     """3 x 3 and 1 x 1 filters over a multiple of 32 channels take a gather whose tap offsets are compile-time
     register choices plus a scalar channel offset; MI355X_CONV_STATIC_TAPS=0 sends the same call through the tap
     table. Both add up the same products in the same order."""
@@ -552,11 +597,9 @@ def test_conv_taps_known_at_compile_time(monkeypatch, shape, wshape, strides, pa
     expected = O.relu(O.conv2d(x, w, b, strides=strides, pads=pads, dilations=dilations))
     tx, tw, tb = (torch.from_numpy(a).cuda() for a in (x, w, b))
     lib = _lib.library()
-    monkeypatch.setenv("MI355X_CONV_GATHER_BN", str(gather_bn))
     results = []
     for setting in ("1", "0"):
-        monkeypatch.setenv("MI355X_CONV_STATIC_TAPS", setting)
-        lib.mi355x_reload_tuning()
+        tuning(MI355X_CONV_GATHER_BN=gather_bn, MI355X_CONV_STATIC_TAPS=setting)
         y = torch.full(expected.shape, float("nan"), device="cuda")
         status = lib.mi355x_conv2d_f32(tx.data_ptr(), tw.data_ptr(), tb.data_ptr(), y.data_ptr(), *shape, wshape[0], wshape[2], wshape[3],
                                        _lib.i64_array(pads), _lib.i64_array(strides), _lib.i64_array(dilations),
@@ -564,9 +607,6 @@ def test_conv_taps_known_at_compile_time(monkeypatch, shape, wshape, strides, pa
         assert status == 0, lib.mi355x_last_error()
         torch.cuda.synchronize()
         results.append(y.cpu().numpy())
-    monkeypatch.delenv("MI355X_CONV_STATIC_TAPS", raising=False)
-    monkeypatch.delenv("MI355X_CONV_GATHER_BN", raising=False)
-    lib.mi355x_reload_tuning()
     assert rel_err(expected, results[0]) < FP32_REL_TOL
     assert np.array_equal(results[0], results[1])
 
