@@ -27,7 +27,7 @@ struct Tuning {
     int gemm_config = -1, gemm_nt_bn = 0, gemm_nt_bk = 0, gemm_group_m = 0;
     int conv_config = -1, conv_gather_bn = 0, conv_tail = -1, conv_static_taps = 1;
     bool mmi_generic = false;
-    int mmi_wgs_per_cu = 0;
+    int mmi_wgs_per_cu = 0, mmi_tile = 0;
 };
 Tuning tuning();   // a copy taken under the lock: a reload never changes what a launch in progress reads
 int device_cus();

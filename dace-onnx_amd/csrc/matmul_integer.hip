@@ -17,6 +17,7 @@
 
 #include <stdlib.h>
 #include <type_traits>
+#include <utility>
 
 namespace mi355x {
 
@@ -32,6 +33,16 @@ struct MMIArgs {
 };
 
 typedef int i32x2 __attribute__((ext_vector_type(2)));
+
+template <class F, int... I>
+__device__ __forceinline__ void mmi_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<0>) ... f(integral_constant<N-1>)
+template <int N, class F>
+__device__ __forceinline__ void mmi_static_for(F&& f) {
+    mmi_static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
 
 // zero point of row m of A / column n of B as the kernels use it: that of the signed bytes they multiply
 __device__ __forceinline__ int32_t a_zero_point(const MMIArgs& p, int64_t m) {
@@ -558,10 +569,17 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     issue_loads(0);
     if (total_steps > 1) issue_loads(1);
     if constexpr (ZP) {
-        // (the aligned word that holds the byte: no conversion instruction, hence no wait, at this point)
-        za_raw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.za_ptr ? p.za_ptr : p.A) & ~(uintptr_t)3);
-        zb_raw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.zb_ptr ? p.zb_ptr : p.B) & ~(uintptr_t)3);
-        MI355X_WAIT_VMCNT(2);   // operations complete in order: the transfers have landed, these two loads may not have
+        // (the aligned word that holds the byte; written as assembly like the transfers, so that exactly two vector
+        // memory operations follow them whatever the compiler would have selected for a wave-uniform address)
+        const uint32_t* za_word = reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.za_ptr ? p.za_ptr : p.A) & ~(uintptr_t)3);
+        const uint32_t* zb_word = reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.zb_ptr ? p.zb_ptr : p.B) & ~(uintptr_t)3);
+        const uint32_t zero = 0u;
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(za_raw) : "v"(zero), "s"(za_word) : "memory");
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(zb_raw) : "v"(zero), "s"(zb_word) : "memory");
+        // operations complete in order: with at most these 2 outstanding the transfers have landed. The two values are first
+        // looked at in finish_tile, behind its own fence and at least one wait of the loop (vmcnt(0), or vmcnt(63) with 64
+        // stores issued after them).
+        MI355X_WAIT_VMCNT(2);
     } else {
         MI355X_WAIT_VMCNT(0);
     }
@@ -606,6 +624,355 @@ __global__ __launch_bounds__(256, (AU && BU) ? 2 : 3) void matmul_integer_i8_str
     if (p.trace) MI355X_WAIT_VMCNT(0);   // slot 3: the last store is acknowledged
 #endif
     MI355X_TRACE_STAMP(p, 3);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same data path with one tile per workgroup and a loop the compiler can count: waves in a WAVES_M x WAVES_N
+// grid, a wave multiplies 64 rows x 32 TNF columns (2 x 2 waves and TNF = 2: 128 x 128 tiles, three workgroups
+// per CU; 4 x 2 waves and TNF = 3: 256 x 192 tiles, one workgroup per CU). What differs from the persistent kernel
+// above is the shape of the code, not of the data: the K loop is unrolled over the NS LDS stages, so every LDS
+// address is a register set up before the loop plus an immediate (no vector arithmetic per step besides the
+// zero-point sums), the loop body has no tile bookkeeping in it, and the result is stored once, behind the loop.
+// The compiler's s_waitcnt for the operand reads is then a count (the reads of the next sub-step stay in flight
+// under the current one's MFMAs) instead of the wait for everything it falls back to in a loop with the stores inside.
+constexpr int mmt_b_swizzle(int krow, int pos, int cpr) {
+    return cpr == 8 ? pos ^ (2 * ((krow >> 1) & 3)) : pos ^ (((krow >> 2) & 1) | (((krow >> 4) & 1) << 1));
+}
+
+template <bool ZP, bool AU, bool BU, int WAVES_M, int WAVES_N, int TNF, int NS, bool A_DIRECT = false>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, WAVES_M * WAVES_N == 4 ? ((AU && BU) ? 2 : 3) : 1) void matmul_integer_i8_tile_kernel(MMIArgs p) {
+    constexpr int BM = 64 * WAVES_M, BN = 32 * TNF * WAVES_N, BK = 64;
+    constexpr int A_STAGE = A_DIRECT ? 0 : BM * BK, STAGE = A_STAGE + BK * BN, NW = WAVES_M * WAVES_N;
+    constexpr int CPR = BN / 16;                              // 16-byte chunks of a B row
+    constexpr int NA = A_DIRECT ? 0 : BM / 16, NT = NA + BN / 16;            // transfer instructions of a step: 1 KB each, A first
+    constexpr int PER_WAVE = (NT + NW - 1) / NW;
+    static_assert(WAVES_N == 2, "row sums are shared by the two waves of a wave row, one sub-step each");
+    static_assert(WAVES_M == 2 || WAVES_M == 4, "column sums are shared by the waves of a wave column, one sub-step in WAVES_M each");
+    static_assert(CPR == 8 || CPR == 12, "swizzle of the B stage");
+    static_assert(NS >= 3, "a stage is overwritten NS - 1 steps after it was read");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[NS * STAGE];
+    __shared__ __attribute__((aligned(16))) int32_t lds_rows[WAVES_M][2][64];   // [wave row][summed by wave column][row]
+    __shared__ int32_t lds_cols[WAVES_N][WAVES_M][32 * TNF];                    // [wave column][summed by wave row][column]
+    const int tid = threadIdx.x;
+    const int lane = tid % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int lj = lane % 32, lg = lane / 32;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int wm0 = wm * 64, wn0 = wn * (32 * TNF);
+
+    MI355X_TRACE_STAMP(p, 0);
+    MI355X_TRACE_HWID(p);
+    const int ktiles = (int)(p.K / BK);
+    const int last_tile = ktiles - 1;
+    int64_t m0, n0;
+    {
+        int64_t tm, tn;
+        tile_coords(xcd_remap(blockIdx.x, p.nwg), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+        m0 = tm * BM;
+        n0 = tn * BN;
+    }
+
+    // ---- loader: transfer instruction q of a step moves 1 KB, 16 bytes per lane: q < NA fills A rows 16 q .. + 15
+    //   (lane i -> row + i / 4, slot i % 4 swizzled), the others fill the B stage (instruction q' = q - NA: chunks
+    //   64 q' .. + 63, chunk c = k-row c / CPR, position c % CPR). Wave w issues q = w, w + NW, ...; where that runs
+    //   past the last instruction, the wave repeats its previous one (same bytes to the same place).
+    // Rows past M and columns past N are clamped into the matrix (what they produce is never stored).
+    const int8_t* const a_tile = p.A + m0 * p.K;
+    const int8_t* const b_tile = p.B + n0;
+    const int64_t b_step = (int64_t)BK * p.N;
+    uint32_t t_off[PER_WAVE];
+    int q_of[PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+        const int q0 = wave + i * NW;
+        const int q = q0 < NT ? q0 : q0 - NW;   // wave-uniform
+        q_of[i] = q;
+        if (q < NA) {
+            int64_t am = m0 + 16 * q + lane / 4;
+            am = am < p.M ? am : p.M - 1;
+            t_off[i] = (uint32_t)((am - m0) * p.K) + 16u * (uint32_t)((lane % 4) ^ ((lane >> 4) & 3));
+        } else {
+            const int c = 64 * (q - NA) + lane, krow = c / CPR, pos = c - CPR * krow;
+            int64_t bn = n0 + 16 * mmt_b_swizzle(krow, pos, CPR);
+            bn = bn < p.N ? bn : p.N - 16;
+            t_off[i] = (uint32_t)krow * (uint32_t)p.N + (uint32_t)(bn - n0);
+        }
+    }
+    const uint32_t lds_base = lds_address(lds);
+    uint32_t t_lds[PER_WAVE];   // where in a stage instruction i of this wave writes (wave-uniform)
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) t_lds[i] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_base + 1024u * (uint32_t)q_of[i]));
+    // k-tile kt of the tile's operands; look-aheads past the end of K fetch the last k-tile again
+    auto issue_loads = [&](int stage, int kt) __attribute__((always_inline)) {
+        const int k = kt < last_tile ? kt : last_tile;
+        const int8_t* const a_base = a_tile + (int64_t)k * BK;
+        const int8_t* const b_base = b_tile + (int64_t)k * b_step;
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) global_to_lds_16(q_of[i] < NA ? a_base : b_base, t_off[i], t_lds[i] + (uint32_t)(stage * STAGE));
+    };
+
+    // ---- operand reads: A operand i is row wm0 + 32 i + lj, chunk 2 ks + lg at (chunk ^ swizzle); B operand t is
+    // columns wn0 + 32 t + lane % 32, lane i16 of a group of 16 addresses k-row 32 ks + 16 lg + i16 / 2 (+ 8 for the
+    // second read), 8 columns from 16 (lane / 16 % 2) + 8 (i16 % 2). One pointer per operand and sub-step, set up here.
+    const uint8_t* a_ptr[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int row = wm0 + 32 * i + lj;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) a_ptr[i][ks] = lds + row * BK + 16 * ((2 * ks + lg) ^ ((row >> 2) & 3));
+    }
+    const int i16 = lane & 15, half = (lane >> 4) & 1, rib = i16 >> 1;
+    const uint8_t* b_ptr[TNF];
+#pragma unroll
+    for (int t = 0; t < TNF; ++t) {
+        const int cc = (wn0 + 32 * t) / 16 + half, krow = 16 * lg + rib;
+        b_ptr[t] = lds + A_STAGE + krow * BN + 16 * mmt_b_swizzle(krow, cc, CPR) + 8 * (i16 & 1);
+    }
+
+    i32x16 acc[2][TNF];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int t = 0; t < TNF; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][t][r] = 0;
+    int32_t rowsum[2] = {0, 0}, colsum[TNF] = {};
+    i32x4 fa[2][2], fb[2][TNF];
+    // A_DIRECT (measurement variant): A never enters LDS; a lane's operand (16 consecutive k of one row) is one raw-buffer
+    // load straight into the register the MFMA reads, NS - 1 steps ahead; the two waves of a wave row fetch the same bytes
+    i32x4 ra[A_DIRECT ? NS : 1][2][2];
+    const int64_t a_rows_left = p.M - m0 - wm0;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(p.A + (m0 + wm0) * p.K), 0, a_rows_left > 0 ? (int)((a_rows_left < 64 ? a_rows_left : 64) * p.K) : 0, 0x00020000);
+    uint32_t a_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a_voff[i] = (uint32_t)(32 * i + lj) * (uint32_t)p.K + 16u * (uint32_t)lg;
+    auto load_a = [&](auto slot_tag, int kt) __attribute__((always_inline)) {
+        constexpr int slot = decltype(slot_tag)::value;
+        if constexpr (A_DIRECT) {
+            const int k = kt < last_tile ? kt : last_tile;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+                    ra[slot][i][ks] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, (int)(a_voff[i] + 32u * ks), k * BK, 0));
+        }
+    };
+    auto read_frags = [&](auto set_tag, int stage, auto ks_tag) __attribute__((always_inline)) {
+        constexpr int set = decltype(set_tag)::value, ks = decltype(ks_tag)::value;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            if constexpr (!A_DIRECT) {
+                fa[set][i] = *reinterpret_cast<const i32x4*>(a_ptr[i][ks] + stage * STAGE);
+                if constexpr (AU) fa[set][i] ^= (int)0x80808080u;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TNF; ++t) {
+            const i32x2 lo = lds_read_tr8(b_ptr[t] + stage * STAGE + 32 * BN * ks);
+            const i32x2 hi = lds_read_tr8(b_ptr[t] + stage * STAGE + 32 * BN * ks + 8 * BN);
+            fb[set][t] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+            if constexpr (BU) fb[set][t] ^= (int)0x80808080u;
+        }
+    };
+    // (wm_tag, wn_tag: this wave's place in the wave grid as constants, see the dispatch below; r = step % NS)
+    auto multiply = [&](auto ks_tag, auto r_tag, auto wm_tag, auto wn_tag) __attribute__((always_inline)) {
+        constexpr int ks = decltype(ks_tag)::value;   // operand set ks holds sub-step ks
+        constexpr int r = decltype(r_tag)::value, WM = decltype(wm_tag)::value, WN = decltype(wn_tag)::value;
+        if constexpr (A_DIRECT) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[ks][i] = ra[r][i][ks];
+                if constexpr (AU) fa[ks][i] ^= (int)0x80808080u;
+            }
+        }
+        if constexpr (ZP && WN == ks) {   // the two waves of a wave row sum one sub-step each
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) rowsum[i] = __builtin_amdgcn_sdot4(fa[ks][i][q], 0x01010101, rowsum[i], false);
+        }
+        if constexpr (ZP && WM == ((2 * r + ks) & (WAVES_M - 1))) {   // sub-step 2 kt + ks of the tile, one wave of the column in turn
+#pragma unroll
+            for (int t = 0; t < TNF; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) colsum[t] = __builtin_amdgcn_sdot4(fb[ks][t][q], 0x01010101, colsum[t], false);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int t = 0; t < TNF; ++t) acc[i][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks][i], fb[ks][t], acc[i][t], 0, 0, 0);
+    };
+
+    // ---- prologue: stages 0 .. NS - 2 on their way, then the aligned 32-bit words that hold the first zero points
+    // (behind the operand transfers, so that a cold page never delays the first step; they are looked at after the
+    // loop). Both as assembly, so that the number of memory operations in flight is what is written here: the waits
+    // below count them.
+    mmi_static_for<NS - 1>([&](auto s_tag) {
+        issue_loads(decltype(s_tag)::value, decltype(s_tag)::value);
+        load_a(s_tag, decltype(s_tag)::value);
+    });
+    uint32_t za_raw = 0u, zb_raw = 0u;
+    if constexpr (ZP) {
+        const uint32_t* za_word = reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.za_ptr ? p.za_ptr : p.A) & ~(uintptr_t)3);
+        const uint32_t* zb_word = reinterpret_cast<const uint32_t*>(reinterpret_cast<uintptr_t>(p.zb_ptr ? p.zb_ptr : p.B) & ~(uintptr_t)3);
+        const uint32_t zero = 0u;
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(za_raw) : "v"(zero), "s"(za_word) : "memory");
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(zb_raw) : "v"(zero), "s"(zb_word) : "memory");
+    }
+    // operations complete in order: once all but the (NS - 3) youngest transfer groups and the two zero-point loads
+    // have completed, stages 0 and 1 are in LDS
+    constexpr int GROUP = PER_WAVE + (A_DIRECT ? 4 : 0);   // memory operations a wave issues per step: transfers, then A loads
+    MI355X_WAIT_VMCNT((NS - 3) * GROUP + (A_DIRECT ? 4 : 0) + (ZP ? 2 : 0));
+    __syncthreads();
+    MI355X_TRACE_STAMP(p, 1);   // the first operands are in LDS
+    MI355X_TRACE_CYCLES(p, 12);
+    read_frags(std::integral_constant<int, 0>{}, 0, std::integral_constant<int, 0>{});
+
+    // ---- K loop. At the top of step kt: stages kt and kt + 1 (mod NS) are in LDS and visible to every wave, operand
+    // set 0 holds (stage kt, first 32 k). The transfer of step kt + NS - 1 goes into the stage step kt - 1 read.
+    // The loop exists once per wave of the wave grid, with the wave's row and column as constants: which operands a
+    // wave adds up for the zero points is then decided at compile time, and a step is straight-line code.
+    static_assert((2 * NS) % WAVES_M == 0, "the wave whose turn it is to sum B depends on the step modulo NS only");
+    auto k_loop = [&](auto wm_tag, auto wn_tag) __attribute__((always_inline)) {
+        auto step = [&](auto r_tag, int kt) __attribute__((always_inline)) {
+            constexpr int r = decltype(r_tag)::value;   // kt % NS
+            issue_loads((r + NS - 1) % NS, kt + NS - 1);
+            load_a(std::integral_constant<int, (r + NS - 1) % NS>{}, kt + NS - 1);
+            read_frags(std::integral_constant<int, 1>{}, r, std::integral_constant<int, 1>{});
+            multiply(std::integral_constant<int, 0>{}, r_tag, wm_tag, wn_tag);
+            read_frags(std::integral_constant<int, 0>{}, (r + 1) % NS, std::integral_constant<int, 0>{});
+            multiply(std::integral_constant<int, 1>{}, r_tag, wm_tag, wn_tag);
+            // the transfer of step kt + 2 has to be in LDS behind the barrier: everything but the NS - 3 youngest groups
+            MI355X_WAIT_VMCNT((NS - 3) * GROUP + (A_DIRECT ? 4 : 0));
+            __syncthreads();
+        };
+        for (int kt0 = 0; kt0 < ktiles; kt0 += NS) {
+            mmi_static_for<NS>([&](auto r_tag) {
+                const int kt = kt0 + decltype(r_tag)::value;
+                if (kt < ktiles) step(r_tag, kt);   // uniform; only the last group can be partial
+            });
+        }
+    };
+    mmi_static_for<NW>([&](auto w_tag) {
+        constexpr int w = decltype(w_tag)::value;
+        if (wave == w) k_loop(std::integral_constant<int, w / WAVES_N>{}, std::integral_constant<int, w % WAVES_N>{});
+    });
+    MI355X_TRACE_STAMP(p, 2);
+    MI355X_TRACE_CYCLES(p, 13);
+    MI355X_WAIT_VMCNT(0);   // look-ahead transfers past the end of K, and the zero points
+    if constexpr (ZP) asm volatile("" : "+v"(za_raw), "+v"(zb_raw));   // nothing derived from them is computed before this wait
+
+    // ---- the sums meet in LDS
+    if constexpr (ZP) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int32_t rs = rowsum[i] + __shfl_xor(rowsum[i], 32, WAVE);
+            if (lg == 0) lds_rows[wm][wn][32 * i + lj] = rs;
+        }
+#pragma unroll
+        for (int t = 0; t < TNF; ++t) {
+            const int32_t cs = colsum[t] + __shfl_xor(colsum[t], 32, WAVE);
+            if (lg == 0) lds_cols[wn][wm][32 * t + lj] = cs;
+        }
+        __syncthreads();
+    }
+
+    // ---- Y = acc - zb[n] rowsum[m] - za[m] (colsum[n] - K zb[n])
+    // the tile's rows as a raw buffer: stores past the last row fall outside it and are dropped, columns
+    // past N are dropped through offset bit 31 (BM rows of N int32 stay below 2^31 bytes: launch precondition)
+    const int64_t rows_left = p.M - m0 < BM ? p.M - m0 : BM;
+    const __amdgpu_buffer_rsrc_t y_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(p.Y + m0 * p.N + n0, 0, (int)((rows_left * p.N - n0) * 4), 0x00020000);
+    const bool one_each = p.za_stride == 0 && p.zb_stride == 0;   // wave-uniform
+    uint32_t za_one = 0u, zb_one = 0u;
+    if constexpr (ZP) {
+        const int32_t a_bias = AU ? 128 : 0, b_bias = BU ? 128 : 0;
+        const uint32_t za_byte = (za_raw >> (8 * (reinterpret_cast<uintptr_t>(p.za_ptr) & 3))) & 0xffu;
+        const uint32_t zb_byte = (zb_raw >> (8 * (reinterpret_cast<uintptr_t>(p.zb_ptr) & 3))) & 0xffu;
+        za_one = (uint32_t)((p.za_ptr ? (AU ? (int32_t)za_byte : (int32_t)(int8_t)za_byte) : 0) - a_bias);
+        zb_one = (uint32_t)((p.zb_ptr ? (BU ? (int32_t)zb_byte : (int32_t)(int8_t)zb_byte) : 0) - b_bias);
+    }
+    const uint32_t row_bytes = (uint32_t)p.N * 4u;
+    uint32_t voff[TNF], zbn[TNF] = {}, c2[TNF] = {};
+#pragma unroll
+    for (int t = 0; t < TNF; ++t) {
+        const int col = wn0 + 32 * t + lj;
+        const bool inside = n0 + col < p.N;
+        voff[t] = (uint32_t)(wm0 + 4 * lg) * row_bytes + (inside ? (uint32_t)col * 4u : 0x80000000u);
+        if constexpr (ZP) {
+            zbn[t] = p.zb_stride == 0 ? zb_one : (inside ? (uint32_t)b_zero_point(p, n0 + col) : 0u);
+            int32_t cs = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES_M; ++w) cs += lds_cols[wn][w][32 * t + lj];
+            c2[t] = (uint32_t)cs - (uint32_t)p.K * zbn[t];
+        }
+    }
+    // 32-bit integer multiplies run at a quarter of the rate of adds: with one zero point per operand the
+    // correction of an element is two subtractions, y = acc - zb rowsum[m] - za (colsum[n] - K zb)
+    uint32_t d_col[TNF] = {};
+    if constexpr (ZP) {
+#pragma unroll
+        for (int t = 0; t < TNF; ++t) d_col[t] = za_one * c2[t];
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        int32_t za_lane = 0;   // zero point of row wm0 + 32 i + lj when there is one per row
+        if constexpr (ZP) {
+            if (p.za_stride != 0) {
+                const int64_t m = m0 + wm0 + 32 * i + lj;
+                za_lane = a_zero_point(p, m < p.M ? m : p.M - 1);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            // row sums of the four rows 32 i + 8 q + 4 lg + e that registers 4 q + e hold
+            i32x4 rs4 = {};
+            if constexpr (ZP)
+                rs4 = *reinterpret_cast<const i32x4*>(&lds_rows[wm][0][32 * i + 8 * q + 4 * lg]) +
+                      *reinterpret_cast<const i32x4*>(&lds_rows[wm][1][32 * i + 8 * q + 4 * lg]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = 4 * q + e;
+                const uint32_t roff = (uint32_t)(32 * i + 8 * q + e) * row_bytes;
+                uint32_t y[TNF];
+#pragma unroll
+                for (int t = 0; t < TNF; ++t) y[t] = (uint32_t)acc[i][t][r];
+                if constexpr (ZP) {
+                    const uint32_t rs = (uint32_t)rs4[e];
+                    if (one_each) {
+                        const uint32_t e_row = zb_one * rs;
+#pragma unroll
+                        for (int t = 0; t < TNF; ++t) y[t] = y[t] - e_row - d_col[t];
+                    } else {
+                        const uint32_t zam = p.za_stride == 0 ? za_one : (uint32_t)__shfl(za_lane, 8 * q + 4 * lg + e, WAVE);
+#pragma unroll
+                        for (int t = 0; t < TNF; ++t) y[t] = y[t] - zbn[t] * rs - zam * c2[t];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < TNF; ++t)
+                    __builtin_amdgcn_raw_buffer_store_b32((int32_t)y[t], y_rsrc, (int)(voff[t] + roff), 0, 0);
+            }
+        }
+    }
+#ifdef MI355X_WG_TRACE
+    if (p.trace) MI355X_WAIT_VMCNT(0);   // slot 3: the last store is acknowledged
+#endif
+    MI355X_TRACE_STAMP(p, 3);
+}
+
+template <bool ZP, int WAVES_M, int WAVES_N, int TNF, int NS, bool A_DIRECT = false>
+static void launch_tile(const MMIArgs& p, hipStream_t st) {
+    const dim3 g((unsigned)p.nwg), b(64 * WAVES_M * WAVES_N);
+    if (p.a_unsigned) {
+        if (p.b_unsigned) hipLaunchKernelGGL((matmul_integer_i8_tile_kernel<true, true, true, WAVES_M, WAVES_N, TNF, NS>), g, b, 0, st, p);
+        else hipLaunchKernelGGL((matmul_integer_i8_tile_kernel<true, true, false, WAVES_M, WAVES_N, TNF, NS>), g, b, 0, st, p);
+    } else if (p.b_unsigned) {
+        hipLaunchKernelGGL((matmul_integer_i8_tile_kernel<true, false, true, WAVES_M, WAVES_N, TNF, NS>), g, b, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((matmul_integer_i8_tile_kernel<ZP, false, false, WAVES_M, WAVES_N, TNF, NS, A_DIRECT>), g, b, 0, st, p);
+    }
 }
 
 template <bool ZP>
@@ -656,6 +1023,38 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
     if (K > 0 && K % MMF_BK == 0 && N % 16 == 0 && al(A, 16) && al(B, 16) && al(Y, 4) && N < ((int64_t)1 << 21) &&
         K < ((int64_t)1 << 24) && !tune.mmi_generic) {
         if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "matmul_integer: no usable HIP device");
+        // Three forms of the same data path. Long K: 256 x 192 tiles, one workgroup of eight waves per CU (0.72 us per 64-k
+        // step of the whole 4096 x 3072 problem against 0.87 us: less LDS traffic per MFMA and 14 instead of 16 zero-point
+        // instructions per wave and step), where such tiles fill the CUs as evenly as 128 x 128 tiles in threes do. Short K:
+        // the persistent kernel below, whose three workgroups per CU hide each other's start and stores (K = 768: 19.2 us
+        // against 19.7 us). MI355X_MMI_TILE forces 128 (one 128 x 128 tile per workgroup) or 256; 129 and 257 are the same
+        // two with A read straight from global memory into the MFMA registers, kept as a measurement (signed operands only):
+        // the vector memory pipe takes a load whose neighbouring lanes touch different rows at one row per cycle, 64 cycles
+        // per instruction instead of 16, and a step takes 1.63 us / 1.06 us.
+        const int64_t wide_tiles = ceil_div(M, (int64_t)256) * ceil_div(N, (int64_t)192);
+        const double narrow_cost = (double)ceil_div(p.nwg, (int64_t)3 * cus) * 3 * 128 * 128;
+        const double wide_cost = (double)ceil_div(wide_tiles, (int64_t)cus) * 256 * 192;
+        const int tile = tune.mmi_tile ? tune.mmi_tile :   // (1: none of the tile kernels)
+                         (K >= 1536 && wide_cost <= narrow_cost && N < ((int64_t)1 << 20)) ? 256 : 0;
+        if (tile == 128 || tile == 256 || tile == 129 || tile == 257) {
+            const bool a_direct = (tile & 1) && !p.a_unsigned && !p.b_unsigned && p.M * p.K < ((int64_t)1 << 31);
+            const int bm = tile >= 256 ? 256 : 128, bn = tile >= 256 ? 192 : 128;
+            p.tiles_m = ceil_div(M, (int64_t)bm);
+            p.tiles_n = ceil_div(N, (int64_t)bn);
+            p.nwg = p.tiles_m * p.tiles_n;
+            const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = (int64_t)(bm == 256 ? 1 : 3) * (cus / NUM_XCD);
+            p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, bm, bn);
+            const bool zp = a_zero_point || b_zero_point;
+            if (a_direct) {
+                if (bm == 256) { if (zp) launch_tile<true, 4, 2, 3, 4, true>(p, st); else launch_tile<false, 4, 2, 3, 4, true>(p, st); }
+                else { if (zp) launch_tile<true, 2, 2, 2, 3, true>(p, st); else launch_tile<false, 2, 2, 2, 3, true>(p, st); }
+            } else if (bm == 256) {
+                if (zp) launch_tile<true, 4, 2, 3, 4>(p, st); else launch_tile<false, 4, 2, 3, 4>(p, st);
+            } else {
+                if (zp) launch_tile<true, 2, 2, 2, 3>(p, st); else launch_tile<false, 2, 2, 2, 3>(p, st);
+            }
+            return check_launch("matmul_integer_i8_tile_kernel");
+        }
         // persistent grid: three workgroups per CU (a multiple of the XCD count), fewer if there are fewer tiles
         int64_t grid = (int64_t)(tune.mmi_wgs_per_cu > 0 ? tune.mmi_wgs_per_cu : 3) * (cus / NUM_XCD) * NUM_XCD;
         if (grid > p.nwg || grid <= 0) grid = p.nwg;

@@ -340,18 +340,43 @@ def test_forced_conv_tile_variants(tuning, config):
     assert rel_err(O.conv2d(x, w, b, pads=(1, 1, 1, 1)), y) < FP32_REL_TOL
 
 
-@pytest.mark.parametrize("variables", [{"MI355X_MMI_GENERIC": 1}, {"MI355X_MMI_WGS_PER_CU": 1}, {"MI355X_MMI_WGS_PER_CU": 2}])
-def test_forced_matmul_integer_variants(tuning, variables):
-    """The generic MatMulInteger kernel on a shape the streaming kernel would take, and the streaming kernel with fewer
-    workgroups per CU than it picks: bit-exact against the int64 formula."""
+@pytest.mark.parametrize("variables", [{"MI355X_MMI_GENERIC": 1}, {"MI355X_MMI_WGS_PER_CU": 1}, {"MI355X_MMI_WGS_PER_CU": 2},
+                                       {"MI355X_MMI_TILE": 128}, {"MI355X_MMI_TILE": 256}, {"MI355X_MMI_TILE": 129},
+                                       {"MI355X_MMI_TILE": 257}])
+@pytest.mark.parametrize("M, N, K", [(384, 272, 192), (300, 208, 64), (1000, 400, 320)])
+def test_forced_matmul_integer_variants(tuning, variables, M, N, K):
+    """Every form of MatMulInteger on shapes the library would give to another one: the generic kernel, the persistent
+    kernel with fewer workgroups per CU, one 128 x 128 or 256 x 192 tile per workgroup, and the two measurement variants
+    that read A straight from global memory. Signed and unsigned operands, one zero point per operand and one per row /
+    column; bit-exact against the int64 formula."""
     tuning(**variables)
-    rng = np.random.default_rng(55)
-    A = rng.integers(-128, 128, size=(384, 192), dtype=np.int8)
-    B = rng.integers(-128, 128, size=(192, 272), dtype=np.int8)
-    Y = np.zeros((384, 272), np.int32)
-    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array(3, np.int8), b_zero_point=np.array(-2, np.int8), Y=Y)
-    want = (A.astype(np.int64) - 3) @ (B.astype(np.int64) + 2)
-    assert np.array_equal(want, Y)
+    lib = _lib.library()
+    rng = np.random.default_rng(55 + M)
+    for a_unsigned, b_unsigned, per_axis in ((0, 0, False), (0, 0, True), (1, 0, False), (0, 1, True), (1, 1, False)):
+        A = rng.integers(0, 256, size=(M, K)).astype(np.uint8) if a_unsigned else rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+        B = rng.integers(0, 256, size=(K, N)).astype(np.uint8) if b_unsigned else rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+        za = rng.integers(0, 100, size=M if per_axis else 1).astype(A.dtype)
+        zb = rng.integers(0, 100, size=N if per_axis else 1).astype(B.dtype)
+        ta, tb, tza, tzb = (torch.from_numpy(v).cuda() for v in (A, B, za, zb))
+        y = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+        _lib.check(lib.mi355x_matmul_integer(ta.data_ptr(), tb.data_ptr(), tza.data_ptr(), tzb.data_ptr(), y.data_ptr(), M, N, K,
+                                             a_unsigned, b_unsigned, za.size, zb.size, _lib.current_stream()), "matmul_integer")
+        want = (A.astype(np.int64) - za.astype(np.int64).reshape(-1, 1)) @ (B.astype(np.int64) - zb.astype(np.int64).reshape(1, -1))
+        assert np.array_equal(want.astype(np.int32), y.cpu().numpy()), (variables, a_unsigned, b_unsigned, per_axis)
+
+
+def test_matmul_integer_long_k_takes_the_wide_tile_and_matches(c_oracle):
+    """K >= 1536 on a shape whose 256 x 192 tiles fill the CUs: the library picks the one-tile-per-workgroup kernel by
+    itself; checked against the C restatement on every element and against the checksum identity."""
+    rng = np.random.default_rng(56)
+    A = rng.integers(-128, 128, size=(2048, 1536), dtype=np.int8)
+    B = rng.integers(-128, 128, size=(1536, 1536), dtype=np.int8)
+    Y = np.zeros((2048, 1536), np.int32)
+    donnx.ONNXMatMulInteger(A=A, B=B, a_zero_point=np.array(-5, np.int8), b_zero_point=np.array(7, np.int8), Y=Y)
+    assert np.array_equal(c_oracle.matmul_integer(A, B, -5, 7), Y)
+    ca = A.astype(np.int64).sum(0) + 5 * 2048
+    rb = B.astype(np.int64).sum(1) - 7 * 1536
+    assert int(Y.astype(np.int64).sum()) == int(ca @ rb)
 
 
 def test_save_transients_keeps_every_intermediate(golden):
