@@ -61,6 +61,7 @@ static void parse_tuning(Tuning& t) {
     t.mmi_generic = getenv("MI355X_MMI_GENERIC") != nullptr;
     t.mmi_wgs_per_cu = env_int("MI355X_MMI_WGS_PER_CU", 0);
     t.mmi_tile = env_int("MI355X_MMI_TILE", 0);
+    t.attn_waves = env_int("MI355X_ATTN_WAVES", 0);
 }
 
 Tuning tuning() {

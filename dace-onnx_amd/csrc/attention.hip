@@ -44,8 +44,13 @@ __device__ __forceinline__ float quad_lanes_sum(float v) {
     return v + __shfl_xor(v, 32, WAVE);
 }
 
-__global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p) {
+// WAVES waves of 16 query rows each per workgroup: 4 (64 rows, two workgroups per 128-row slice) is what the library
+// uses; 3 and 2 (48 and 32 rows: three and four workgroups per slice, the last one of three with two working waves)
+// exist to measure whether more, smaller workgroups help, see MI355X_ATTN_WAVES in the launcher.
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attention_f32_kernel(AttnArgs p) {
     constexpr int SK = AT_SK, D = AT_D, PITCH = AT_PITCH, NJ = SK / 16, NC = D / 16;
+    constexpr int NT = 64 * WAVES, VECS = SK * D / 4, PER_T = (VECS + NT - 1) / NT;   // K / V tile: 16-byte vectors per thread
     __shared__ __attribute__((aligned(16))) float lds_k[SK * PITCH];
     __shared__ __attribute__((aligned(16))) float lds_v[SK * PITCH];
 
@@ -61,14 +66,14 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p) {
     const float* __restrict__ K = p.K + b0 * p.k_sb0 + b1 * p.k_sb1;
     const float* __restrict__ V = p.V + b0 * p.v_sb0 + b1 * p.v_sb1;
     float* __restrict__ O = p.O + b0 * p.o_sb0 + b1 * p.o_sb1;
-    const int64_t q0 = qb * AT_BQ + 16 * wave;   // first query row of this wave
+    const int64_t q0 = qb * (16 * WAVES) + 16 * wave;   // first query row of this wave
 
-    // ---- loads: K and V tiles (8 + 8 vectors per thread), Q operands (4 per lane) ----------------
-    f32x4 rk[8], rv[8], rq[NC];
+    // ---- loads: K and V tiles (PER_T + PER_T vectors per thread), Q operands (4 per lane) ----------------
+    f32x4 rk[PER_T], rv[PER_T], rq[NC];
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int idx = tid + it * 256, row = idx / (D / 4), c4 = idx % (D / 4);
-        rk[it] = *reinterpret_cast<const f32x4*>(K + row * p.k_sr + 4 * c4);
+    for (int it = 0; it < PER_T; ++it) {
+        const int idx = tid + it * NT, row = idx / (D / 4), c4 = idx % (D / 4);
+        if (VECS % NT == 0 || idx < VECS) rk[it] = *reinterpret_cast<const f32x4*>(K + row * p.k_sr + 4 * c4);
     }
     {
         int64_t qrow = q0 + li;
@@ -77,19 +82,19 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(AttnArgs p) {
         for (int c = 0; c < NC; ++c) rq[c] = *reinterpret_cast<const f32x4*>(Q + qrow * p.q_sr + 16 * c + 4 * lq);
     }
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int idx = tid + it * 256, row = idx / (D / 4), c4 = idx % (D / 4);
-        rv[it] = *reinterpret_cast<const f32x4*>(V + row * p.v_sr + 4 * c4);
+    for (int it = 0; it < PER_T; ++it) {
+        const int idx = tid + it * NT, row = idx / (D / 4), c4 = idx % (D / 4);
+        if (VECS % NT == 0 || idx < VECS) rv[it] = *reinterpret_cast<const f32x4*>(V + row * p.v_sr + 4 * c4);
     }
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int idx = tid + it * 256, row = idx / (D / 4), c4 = idx % (D / 4);
-        *reinterpret_cast<f32x4*>(lds_k + row * PITCH + 4 * c4) = rk[it];
+    for (int it = 0; it < PER_T; ++it) {
+        const int idx = tid + it * NT, row = idx / (D / 4), c4 = idx % (D / 4);
+        if (VECS % NT == 0 || idx < VECS) *reinterpret_cast<f32x4*>(lds_k + row * PITCH + 4 * c4) = rk[it];
     }
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int idx = tid + it * 256, row = idx / (D / 4), c4 = idx % (D / 4);
-        *reinterpret_cast<f32x4*>(lds_v + row * PITCH + 4 * c4) = rv[it];
+    for (int it = 0; it < PER_T; ++it) {
+        const int idx = tid + it * NT, row = idx / (D / 4), c4 = idx % (D / 4);
+        if (VECS % NT == 0 || idx < VECS) *reinterpret_cast<f32x4*>(lds_v + row * PITCH + 4 * c4) = rv[it];
     }
     __syncthreads();
     if (q0 >= p.Sq) return;  // whole wave beyond the last query row (after the only barrier)
@@ -318,7 +323,17 @@ extern "C" int mi355x_attention_f32(const float* Q, const float* K, const float*
     p.o_sb0 = o_strides[0]; p.o_sb1 = o_strides[1]; p.o_sr = o_strides[2];
     p.scale = scale;
     if (Sk == AT_SK) {
-        hipLaunchKernelGGL(attention_f32_kernel, dim3((unsigned)p.nwg), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        // MI355X_ATTN_WAVES = 2 / 3: 32 / 48 query rows per workgroup instead of 64 (measured on 8 x 12 slices of 128 rows:
+        // 384 / 288 workgroups instead of 192 -- no faster, the time is one wave's chain of loads, 256 MFMAs and stores)
+        const int waves = tuning().attn_waves == 2 || tuning().attn_waves == 3 ? tuning().attn_waves : 4;
+        p.q_blocks = ceil_div(Sq, (int64_t)16 * waves);
+        p.nwg = batch0 * batch1 * p.q_blocks;
+        MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "attention: grid too large");
+        const dim3 g((unsigned)p.nwg);
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        if (waves == 2) hipLaunchKernelGGL(attention_f32_kernel<2>, g, dim3(128), 0, st, p);
+        else if (waves == 3) hipLaunchKernelGGL(attention_f32_kernel<3>, g, dim3(192), 0, st, p);
+        else hipLaunchKernelGGL(attention_f32_kernel<4>, g, dim3(256), 0, st, p);
         return check_launch("attention_f32_kernel");
     }
     hipLaunchKernelGGL(attention_f32_blocks_kernel, dim3((unsigned)p.nwg), dim3(256), 0, static_cast<hipStream_t>(stream), p);

@@ -28,6 +28,7 @@ struct Tuning {
     int conv_config = -1, conv_gather_bn = 0, conv_tail = -1, conv_static_taps = 1;
     bool mmi_generic = false;
     int mmi_wgs_per_cu = 0, mmi_tile = 0;
+    int attn_waves = 0;
 };
 Tuning tuning();   // a copy taken under the lock: a reload never changes what a launch in progress reads
 int device_cus();

@@ -251,7 +251,8 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     MI355X_REQUIRE(p.nwg < ((int64_t)1 << 31), "gemm: grid too large (%lld workgroups)", (long long)p.nwg);
     {   // about two workgroups of these tiles share a CU
         const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = 2 * (cus / NUM_XCD);
-        p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, tc.bm, tc.bn);
+        const int64_t per_batch = p.tiles_m * p.tiles_n;   // tiles are numbered batch entry by batch entry
+        p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, resident, tc.bm, tc.bn, K * 4);
     }
     launch_config(cfg, p, a_kc, b_kc, vec, static_cast<hipStream_t>(stream));
     return check_launch("gemm_f32_kernel");

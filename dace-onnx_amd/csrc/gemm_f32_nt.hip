@@ -305,7 +305,8 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.nwg >= ((int64_t)1 << 31)) return false;
     // one workgroup per CU at a time: an XCD holds cus / 8 tiles
     const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD);
-    p.group_m = choose_group_m(p.tiles_m, per_xcd < cus / NUM_XCD ? per_xcd : cus / NUM_XCD, cands[best].bm, cands[best].bn);
+    const int64_t per_batch = p.tiles_m * p.tiles_n;   // tiles are numbered batch entry by batch entry
+    p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, cus / NUM_XCD, cands[best].bm, cands[best].bn, p.K * 4);
     if (tune.gemm_group_m > 0) p.group_m = tune.gemm_group_m;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
     // The smallest variant walks K in 64-k tiles with a three-deep ring where K allows: half the barriers per FLOP

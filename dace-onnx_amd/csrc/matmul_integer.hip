@@ -1043,7 +1043,7 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
             p.tiles_n = ceil_div(N, (int64_t)bn);
             p.nwg = p.tiles_m * p.tiles_n;
             const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = (int64_t)(bm == 256 ? 1 : 3) * (cus / NUM_XCD);
-            p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, bm, bn);
+            p.group_m = choose_group_m(p.tiles_m, per_xcd, resident, bm, bn, K);
             const bool zp = a_zero_point || b_zero_point;
             if (a_direct) {
                 if (bm == 256) { if (zp) launch_tile<true, 4, 2, 3, 4, true>(p, st); else launch_tile<false, 4, 2, 3, 4, true>(p, st); }
@@ -1059,7 +1059,7 @@ extern "C" int mi355x_matmul_integer(const void* A, const void* B, const void* a
         int64_t grid = (int64_t)(tune.mmi_wgs_per_cu > 0 ? tune.mmi_wgs_per_cu : 3) * (cus / NUM_XCD) * NUM_XCD;
         if (grid > p.nwg || grid <= 0) grid = p.nwg;
         const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD), resident = ceil_div(grid, (int64_t)NUM_XCD);
-        p.group_m = choose_group_m(p.tiles_m, per_xcd < resident ? per_xcd : resident, MMF_BM, MMF_BN);
+        p.group_m = choose_group_m(p.tiles_m, per_xcd, resident, MMF_BM, MMF_BN, K);
         if (a_zero_point || b_zero_point) launch_stream<true>(p, grid, st);
         else launch_stream<false>(p, grid, st);
         return check_launch("matmul_integer_i8_stream_kernel");

@@ -209,9 +209,12 @@ def test_layer_normalization(shape, axis):
     assert rel_err(O.layer_normalization(X, g, None, axis=axis, epsilon=1e-5), Y2) < FP32_REL_TOL
 
 
+@pytest.mark.parametrize("waves", [None, 2, 3])
 @pytest.mark.parametrize("batch, sq", [((2, 3), 128), ((1, 5), 100), ((4, ), 16), ((1, 1), 1)])
-def test_fused_attention_c_abi(batch, sq):
-    # softmax(scale * Q K^T) V through the C ABI, operands as strided slices of one packed projection
+def test_fused_attention_c_abi(tuning, batch, sq, waves):
+    # softmax(scale * Q K^T) V through the C ABI, operands as strided slices of one packed projection; with the
+    # library's 64 query rows per workgroup and with the 32- and 48-row forms MI355X_ATTN_WAVES selects
+    tuning(MI355X_ATTN_WAVES=waves)
     rng = np.random.default_rng(31)
     b0, b1 = (1, ) * (2 - len(batch)) + tuple(batch)
     packed = torch.from_numpy(rng.normal(size=(b0, max(sq, 128), b1, 3, 64)).astype(np.float32)).cuda()
