@@ -24,4 +24,7 @@ struct GemmArgs {
 // the problem is outside what that kernel handles (nothing launched).
 bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream);
 
+// GEMM with both operands contiguous along k whose eight waves split K (gemm_f32_ksplit.hip): 32 x 96 tiles.
+bool launch_gemm_f32_ksplit(GemmArgs p, int cus, hipStream_t stream);
+
 }  // namespace mi355x

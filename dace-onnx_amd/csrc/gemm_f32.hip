@@ -241,8 +241,13 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "gemm: no usable HIP device");
     // both operands contiguous along k (activations x pre-transposed weights, Q K^T):
     // the dedicated kernel reads every MFMA fragment with 16-byte accesses
-    if (a_kc && b_kc && vec && tuning().gemm_config < 0 && launch_gemm_f32_nt(p, cus, static_cast<hipStream_t>(stream)))
-        return check_launch("gemm_f32_nt_kernel");
+    const Tuning tune = tuning();
+    if (a_kc && b_kc && vec && tune.gemm_config < 0) {
+        // MI355X_GEMM_KSPLIT: 1 sends every such product to the kernel whose waves split K, 0 none
+        if (tune.gemm_ksplit == 1 && launch_gemm_f32_ksplit(p, cus, static_cast<hipStream_t>(stream)))
+            return check_launch("gemm_f32_ksplit_kernel");
+        if (launch_gemm_f32_nt(p, cus, static_cast<hipStream_t>(stream))) return check_launch("gemm_f32_nt_kernel");
+    }
     const int cfg = choose_config(batch, M, N, K, cus);
     const TileConfig& tc = kConfigs[cfg];
     p.tiles_m = ceil_div(M, tc.bm);

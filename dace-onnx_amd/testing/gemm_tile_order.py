@@ -6,7 +6,8 @@
 
 ``MI355X_GEMM_GROUP_M`` sets the height, in tile rows, of the panels an XCD's slab of tiles is walked in (the library's
 own choice makes the block of tiles resident on an XCD about square in operand bytes); ``MI355X_GEMM_CONFIG`` sends the
-problem to the generic kernel, which stages both operands through LDS. With ``--dispatch n`` every combination is
+problem to the generic kernel, which stages both operands through LDS; ``MI355X_GEMM_KSPLIT=1`` to the kernel whose eight
+waves split K (``csrc/gemm_f32_ksplit.hip``). With ``--dispatch n`` every combination is
 launched ``n`` times back to back, in the order printed, so that a per-dispatch counter file can be read by position.
 """
 import argparse
@@ -20,6 +21,7 @@ WALKS = (("library", {}), ("group_m 1", {"MI355X_GEMM_GROUP_M": "1"}), ("group_m
          ("group_m 3", {"MI355X_GEMM_GROUP_M": "3"}), ("group_m 4", {"MI355X_GEMM_GROUP_M": "4"}),
          ("group_m 6", {"MI355X_GEMM_GROUP_M": "6"}), ("group_m 8", {"MI355X_GEMM_GROUP_M": "8"}),
          ("group_m 16", {"MI355X_GEMM_GROUP_M": "16"}),
+         ("k split over 8 waves, 32x96 tiles, 32x32x2 MFMA", {"MI355X_GEMM_KSPLIT": "1"}),
          ("generic 64x48 (both operands through LDS)", {"MI355X_GEMM_CONFIG": "2"}),
          ("generic 128x128 (both operands through LDS)", {"MI355X_GEMM_CONFIG": "0"}))
 
@@ -39,7 +41,7 @@ def main():
                                              _lib.i64_array([0, 0, K, 1]), _lib.i64_array([0, 0, 1, K]), _lib.i64_array([0, 0, N]),
                                              _lib.i64_array([0, 0, N]), 1.0, epi, st())
         for walk, variables in WALKS:
-            for key in ("MI355X_GEMM_GROUP_M", "MI355X_GEMM_CONFIG"):
+            for key in ("MI355X_GEMM_GROUP_M", "MI355X_GEMM_CONFIG", "MI355X_GEMM_KSPLIT"):
                 os.environ.pop(key, None)
             os.environ.update(variables)
             lib.mi355x_reload_tuning()
@@ -51,7 +53,7 @@ def main():
                 index += args.dispatch
             else:
                 print(f"{name:5s} {M}x{N}x{K:<5d} {walk:46s} {graph_time_us(launch, reps=20):8.2f} us", flush=True)
-    for key in ("MI355X_GEMM_GROUP_M", "MI355X_GEMM_CONFIG"):
+    for key in ("MI355X_GEMM_GROUP_M", "MI355X_GEMM_CONFIG", "MI355X_GEMM_KSPLIT"):
         os.environ.pop(key, None)
     lib.mi355x_reload_tuning()
 

@@ -5,7 +5,7 @@ into the convolution, k-contiguous GEMM and MatMulInteger kernels (start of a wo
 main loop, end of the workgroup, hardware id of its CU). This script runs one of the benchmark shapes through that
 build and prints the phases; the package itself never loads the trace build.
 
-    python -m dace_onnx_amd.testing.wg_trace conv4 | mmi5 | qkv | out | ffn1 | ffn2
+    python -m dace_onnx_amd.testing.wg_trace conv4 | mmi5 | qkv | out | ffn1 | ffn2 | out_ksplit | ffn2_ksplit
 
 What the stamps mean per kernel (microseconds; the wall clock ticks at 100 MHz):
 
@@ -69,8 +69,16 @@ def _workloads(lib, torch):
                                                 _lib.i64_array([0, 0, N]), _lib.i64_array([0, 0, N]), 1.0, epi, st())), (a, w, bias, res, out)
         return make
 
+    def ksplit(make):   # the same GEMM through the kernel whose eight waves split K (MI355X_GEMM_KSPLIT=1)
+        def wrapped():
+            os.environ["MI355X_GEMM_KSPLIT"] = "1"
+            lib.mi355x_reload_tuning()
+            return make()
+        return wrapped
+
     return {"conv4": conv4, "mmi5": mmi5, "qkv": gemm(1024, 2304, 768, 1), "out": gemm(1024, 768, 768, 9),
-            "ffn1": gemm(1024, 3072, 768, 5), "ffn2": gemm(1024, 768, 3072, 9)}
+            "ffn1": gemm(1024, 3072, 768, 5), "ffn2": gemm(1024, 768, 3072, 9),
+            "out_ksplit": ksplit(gemm(1024, 768, 768, 9)), "ffn2_ksplit": ksplit(gemm(1024, 768, 3072, 9))}
 
 
 def trace(name: str, warm_launches: int = 500, max_workgroups: int = 65536):

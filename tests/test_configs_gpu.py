@@ -270,13 +270,16 @@ def test_strided_gemm_head_split_merge_without_copies():
 
 
 # ----------------------------------------------------------------------------- GEMM kernel variants, ragged shapes
-@pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144"])
+@pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144", "ksplit"])
 @pytest.mark.parametrize("M, N, K, epi", [(64, 48, 32, 0), (1, 4, 32, 1), (130, 52, 64, 9), (257, 100, 96, 5), (200, 148, 160, 3),
                                           (1024, 768, 768, 9), (63, 764, 224, 8), (100, 52, 2112, 9)])   # last: 64-k tiles
 def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
     """Both operands k-contiguous (activations x [N, K] weights): every tile variant of that kernel on shapes that
     leave partial tiles in M and N, with each epilogue combination (1 bias, 2 relu, 4 gelu, 8 residual) and alpha."""
-    tuning(MI355X_GEMM_NT_BN=None if tile == "auto" else tile)   # the variables are read once; the fixture reloads them
+    if tile == "ksplit":   # 32 x 96 tiles, the eight waves of a workgroup split K (K = 32 and 64: some waves get no slice)
+        tuning(MI355X_GEMM_KSPLIT=1)
+    else:
+        tuning(MI355X_GEMM_NT_BN=None if tile == "auto" else tile)   # the variables are read once; the fixture reloads them
     lib = _lib.library()
     rng = np.random.default_rng(M * 7 + N * 3 + K + epi)
     a = torch.from_numpy(rng.normal(size=(2, M, K)).astype(np.float32)).cuda()
@@ -302,7 +305,7 @@ def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
 
 @pytest.mark.parametrize("variables", [{"MI355X_GEMM_CONFIG": c} for c in range(5)] + [{"MI355X_GEMM_NT_BK": 32},
                                                                                         {"MI355X_GEMM_NT_BK": 32, "MI355X_GEMM_NT_BN": 64},
-                                                                                        {"MI355X_GEMM_GROUP_M": 1}])
+                                                                                        {"MI355X_GEMM_GROUP_M": 1}, {"MI355X_GEMM_KSPLIT": 1}])
 @pytest.mark.parametrize("M, N, K, epi", [(130, 100, 64, 9), (257, 52, 2112, 5)])
 def test_forced_gemm_variants(tuning, variables, M, N, K, epi):
     """Every tile shape of the generic double-buffered kernel (which the library itself only picks for operands that are
