@@ -660,12 +660,25 @@ class CompiledSDFG:
         # directly (the source, a transient, becomes a view of the caller's buffer). Walking the aliases backwards
         # carries this through chains of them. What cannot be redirected (the source is caller-owned too, or
         # already a view of something else) is copied on the device.
+        # The redirect moves the write of the caller's buffer from the alias's place in the plan to the producer's,
+        # which is earlier: it is only taken when nothing before the alias reads that buffer (an array that is both
+        # an input of an earlier node and the reshaped output keeps its old contents until the copy).
+        def read_before(position, key):
+            for earlier in self._plan[:position]:
+                if earlier[0] == "alias":
+                    if earlier[1] == key:
+                        return True
+                elif any(earlier[2].get(c) == key for c in earlier[1].in_connectors):
+                    return True
+            return False
+
         redirected = set()
-        for item in reversed(self._plan):
+        for position in range(len(self._plan) - 1, -1, -1):
+            item = self._plan[position]
             if item[0] != "alias":
                 continue
             _, src_key, dst_key, _ = item
-            if dst_key in env and src_key not in env and src_key in self._transients:
+            if dst_key in env and src_key not in env and src_key in self._transients and not read_before(position, dst_key):
                 env[src_key] = env[dst_key].reshape(self._transients[src_key].shape)
                 redirected.add((src_key, dst_key))
         for item in self._plan:
@@ -834,12 +847,13 @@ class CompiledSDFG:
                  f'extern "C" int __program_{name}(void** __arrays, void* __dace_current_stream) {{']
         for item in self._plan:
             if item[0] == "alias":
-                _, src_key, dst_key, _ = item
+                _, src_key, dst_key, dst_desc = item
                 if dst_key in self._external:
                     raise NotImplementedError(f"alias into caller-owned array '{dst_key}' needs a device copy")
                 if dst_key not in index:
                     index[dst_key] = len(arrays)
                     arrays.append(dst_key)
+                desc_of[dst_key] = dst_desc   # the view's own element type (an int64 or int8 view is not a float*)
                 lines.append(f"    __arrays[{index[dst_key]}] = __arrays[{index[src_key]}];  // {dst_key} is a view of {src_key}")
                 continue
             _, node, conn_to_key = item

@@ -667,6 +667,40 @@ def test_outputs_that_are_inputs_or_weights():
     assert np.array_equal(donnx.ONNXModel("empty", H.make_model(g0, opset_imports=[H.make_opsetid("", 12)]))(x), x)
 
 
+def test_view_into_a_callers_buffer_that_is_read_earlier():
+    """A transient whose reshaped view is a caller-owned array is normally produced straight into that array. Not when
+    something reads the array before the view is taken: state 1 computes t = -x and y1 = relu(buf), state 2 makes buf the
+    reshaped t. y1 must see what the caller passed in buf, and buf must hold -x afterwards."""
+    from dace_onnx_amd.util import utils
+    sdfg = dace.SDFG("read_then_view")
+    for name, shape in (("x", [2, 3]), ("buf", [3, 2]), ("y1", [3, 2])):
+        sdfg.add_array(name, shape, dace.float32)
+    sdfg.add_transient("t", [2, 3], dace.float32)
+    s1 = sdfg.add_state("compute")
+    neg, relu = donnx.ONNXNeg("neg"), donnx.ONNXRelu("relu")
+    for node, src, dst in ((neg, "x", "t"), (relu, "buf", "y1")):
+        node.add_in_connector("X")
+        node.add_out_connector("Y")
+        s1.add_edge(s1.add_read(src), None, node, "X", sdfg.make_array_memlet(src))
+        s1.add_edge(node, "Y", s1.add_write(dst), None, sdfg.make_array_memlet(dst))
+    s2 = sdfg.add_state("view")
+    alias = dace.AliasNode("reshape", "data", "reshaped")
+    s2.add_edge(s2.add_read("t"), None, alias, "data", sdfg.make_array_memlet("t"))
+    s2.add_edge(alias, "reshaped", s2.add_write("buf"), None, sdfg.make_array_memlet("buf"))
+    utils.expand_onnx_nodes(sdfg)
+    compiled = dace.CompiledSDFG(sdfg)
+    assert [item[0] for item in compiled._plan] == ["call", "call", "alias"]
+    rng = np.random.default_rng(21)
+    x = torch.from_numpy(rng.normal(size=(2, 3)).astype(np.float32)).cuda()
+    buf = torch.from_numpy(rng.normal(size=(3, 2)).astype(np.float32)).cuda()
+    before = buf.clone()
+    y1 = torch.full((3, 2), float("nan"), device="cuda")
+    compiled(x=x, buf=buf, y1=y1)
+    torch.cuda.synchronize()
+    assert torch.equal(y1, torch.relu(before))
+    assert torch.equal(buf, (-x).reshape(3, 2))
+
+
 def test_conv_network_hip_graph_replays_match_eager():
     """A convolution network (Conv+BatchNormalization+Relu folded, MaxPool through LDS, residual epilogue, global
     average pooling, Gemm, LogSoftmax) replayed as one HIP graph: every replay, with eager work and synchronisation

@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 
 import dace_onnx_amd.onnx as donnx
+from dace_onnx_amd.onnx import proto
 from dace_onnx_amd import sdfg as dace
 from dace_onnx_amd.testing.graphs import bert_encoder_layer_model
 from dace_onnx_amd.util import utils
@@ -91,6 +92,23 @@ def test_generated_program_compiles_against_the_header(tmp_path):
         sdfg = make()
         source, _ = dace.CompiledSDFG(sdfg).program_source()
         _build(source, sdfg.name, str(tmp_path), syntax_only=True)
+
+
+def test_integer_view_keeps_its_element_type(tmp_path):
+    """A Reshape of an int32 result is a view (no launch); the tasklet that reads it declares the view with the
+    view's own element type, not as float*."""
+    H, T = proto.helper, proto.TensorProto
+    nodes = [H.make_node("MatMulInteger", ["a", "b"], ["y"]), H.make_node("Reshape", ["y", "shape"], ["yr"]),
+             H.make_node("Cast", ["yr"], ["out"], to=1)]
+    g = H.make_graph(nodes, "g", [H.make_tensor_value_info("a", T.INT8, [64, 128]), H.make_tensor_value_info("b", T.INT8, [128, 48])],
+                     [H.make_tensor_value_info("out", T.FLOAT, [48, 64])],
+                     initializer=[proto.numpy_helper.from_array(np.array([48, 64], np.int64), "shape")])
+    model = donnx.ONNXModel("intview", H.make_model(g, opset_imports=[H.make_opsetid("", 12)]))
+    source, _ = dace.CompiledSDFG(model.expand()).program_source("intview")
+    assert "// yr is a view of y" in source
+    cast = source[source.index("// Cast"):]
+    assert "int32_t* _input = (int32_t*)" in cast and "float* _input" not in cast
+    _build(source, "intview", str(tmp_path), syntax_only=True)
 
 
 def _run_program(compiled, name, tensors, tmp_path):
