@@ -283,30 +283,39 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.K % NT_BK != 0 || p.K == 0) return false;
     // rows are addressed with 32-bit byte offsets from the start of a batch's matrix
     if (p.a_sm < 0 || p.b_sn < 0 || (p.M - 1) * p.a_sm + p.K >= ((int64_t)1 << 29) || (p.N - 1) * p.b_sn + p.K >= ((int64_t)1 << 29)) return false;
-    // Candidates: 64x48, 64x64 and 64x144 tiles with two k-split groups, 128x96 tiles without.
-    // Cost ~ rounds of workgroups over the CUs x tile area, the large tile discounted
-    // for needing half the L2 traffic per FLOP and no reduction.
-    struct Cand { int bm, bn; double weight; };
+    // Candidates: 64x48, 64x64 and 64x144 tiles with two k-split groups, 128x48 and 128x96 tiles without.
+    // Cost ~ rounds of workgroups over the CUs x tile area. 128 x 48 tiles run two workgroups per CU (116 registers), and
+    // two workgroups that share a CU drift apart: one's first loads, last stores and barrier waits run under the other's
+    // MFMAs. Measured against 128 x 96 tiles, one workgroup per CU: 1024 x 3072 x 768 (with Gelu) 42.5 against 43.7 us,
+    // 2048 x 3072 x 768 78.7 against 82.6 us, 4096 x 4096 x 1024 261.8 against 297.5 us (131 TFLOP/s). A 128 x 48 tile
+    // that has a CU to itself loses to two 64 x 48 tiles (512 x 3072 x 768: 24.0 against 23.4 us), hence rounds counted in
+    // pairs for it. 128 x 96 stays selectable by hand (MI355X_GEMM_NT_BN=96).
+    struct Cand { int bm, bn, per_cu; double weight; };
     // (1024 x 2304 x 768, measured: 768 tiles of 64 x 48, two workgroups sharing a CU, 35.2 us; 256 tiles of 64 x 144 36.1 us:
     // the wide tile gets no discount)
-    const Cand cands[] = {{64, 48, 1.0}, {64, 64, 1.0}, {128, 96, 0.8}, {64, 144, 1.0}};
+    const Cand cands[] = {{64, 48, 1, 1.0}, {64, 64, 1, 1.0}, {128, 96, 1, 0.8}, {64, 144, 1, 1.0}, {128, 48, 2, 0.78}};
     int best = 0;
     double best_cost = 1e300;
     const Tuning tune = tuning();
-    const int force = tune.gemm_nt_bn;
-    for (int c = 0; c < 4; ++c) {
+    const int force = tune.gemm_nt_bn, force_bm = tune.gemm_nt_bm;
+    for (int c = 0; c < 5; ++c) {
         const int64_t nwg = p.batch * ceil_div(p.M, cands[c].bm) * ceil_div(p.N, cands[c].bn);
-        const double cost = (double)ceil_div(nwg, (int64_t)cus) * cands[c].bm * cands[c].bn * cands[c].weight;
-        if (force ? force == cands[c].bn : cost < best_cost) { best = c; best_cost = cost; if (force) break; }
+        const double cost = (double)ceil_div(nwg, (int64_t)cus * cands[c].per_cu) * cands[c].per_cu * cands[c].bm * cands[c].bn * cands[c].weight;
+        if (force) {   // MI355X_GEMM_NT_BN picks the tile width, MI355X_GEMM_NT_BM the height where two candidates share a width
+            if (force == cands[c].bn && (force_bm ? force_bm == cands[c].bm : cands[c].bm == 64 || cands[c].bn == 96)) { best = c; break; }
+        } else if (cost < best_cost) {
+            best = c;
+            best_cost = cost;
+        }
     }
     p.tiles_m = ceil_div(p.M, cands[best].bm);
     p.tiles_n = ceil_div(p.N, cands[best].bn);
     p.nwg = p.batch * p.tiles_m * p.tiles_n;
     if (p.nwg >= ((int64_t)1 << 31)) return false;
-    // one workgroup per CU at a time: an XCD holds cus / 8 tiles
+    // an XCD holds cus / 8 tiles at a time (twice that for the candidates that run in pairs)
     const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD);
     const int64_t per_batch = p.tiles_m * p.tiles_n;   // tiles are numbered batch entry by batch entry
-    p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, cus / NUM_XCD, cands[best].bm, cands[best].bn, p.K * 4);
+    p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, (int64_t)cands[best].per_cu * (cus / NUM_XCD), cands[best].bm, cands[best].bn, p.K * 4);
     if (tune.gemm_group_m > 0) p.group_m = tune.gemm_group_m;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
     // The smallest variant walks K in 64-k tiles with a three-deep ring where K allows: half the barriers per FLOP
@@ -319,6 +328,8 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
     else if (best == 2) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
+    else if (best == 4 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1, 64, 3>), grid, block, 0, stream, p);
+    else if (best == 4) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((gemm_f32_nt_kernel<9, 4, 2>), grid, block, 0, stream, p);
     return true;
 }

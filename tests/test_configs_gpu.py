@@ -270,7 +270,7 @@ def test_strided_gemm_head_split_merge_without_copies():
 
 
 # ----------------------------------------------------------------------------- GEMM kernel variants, ragged shapes
-@pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144", "ksplit"])
+@pytest.mark.parametrize("tile", ["auto", "48", "64", "96", "144", "128x48", "ksplit"])
 @pytest.mark.parametrize("M, N, K, epi", [(64, 48, 32, 0), (1, 4, 32, 1), (130, 52, 64, 9), (257, 100, 96, 5), (200, 148, 160, 3),
                                           (1024, 768, 768, 9), (63, 764, 224, 8), (100, 52, 2112, 9)])   # last: 64-k tiles
 def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
@@ -278,6 +278,8 @@ def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
     leave partial tiles in M and N, with each epilogue combination (1 bias, 2 relu, 4 gelu, 8 residual) and alpha."""
     if tile == "ksplit":   # 32 x 96 tiles, the eight waves of a workgroup split K (K = 32 and 64: some waves get no slice)
         tuning(MI355X_GEMM_KSPLIT=1)
+    elif tile == "128x48":
+        tuning(MI355X_GEMM_NT_BM=128, MI355X_GEMM_NT_BN=48)
     else:
         tuning(MI355X_GEMM_NT_BN=None if tile == "auto" else tile)   # the variables are read once; the fixture reloads them
     lib = _lib.library()
@@ -305,7 +307,8 @@ def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
 
 @pytest.mark.parametrize("variables", [{"MI355X_GEMM_CONFIG": c} for c in range(5)] + [{"MI355X_GEMM_NT_BK": 32},
                                                                                         {"MI355X_GEMM_NT_BK": 32, "MI355X_GEMM_NT_BN": 64},
-                                                                                        {"MI355X_GEMM_GROUP_M": 1}, {"MI355X_GEMM_KSPLIT": 1}])
+                                                                                        {"MI355X_GEMM_GROUP_M": 1}, {"MI355X_GEMM_KSPLIT": 1},
+                                       {"MI355X_GEMM_NT_BM": 128, "MI355X_GEMM_NT_BN": 48, "MI355X_GEMM_NT_BK": 32}])
 @pytest.mark.parametrize("M, N, K, epi", [(130, 100, 64, 9), (257, 52, 2112, 5)])
 def test_forced_gemm_variants(tuning, variables, M, N, K, epi):
     """Every tile shape of the generic double-buffered kernel (which the library itself only picks for operands that are
