@@ -50,8 +50,8 @@ constexpr int NT_BK = 32, NT_THREADS = 512, NT_RING = 6, NT_STAGES = 3;
 // (4, 2) for problems with few tiles, (8, 1) for 128-row tiles without a reduction.
 // BK: k extent of a tile (32, or 64 where registers allow: half as many barriers per FLOP); RING: k-tiles in
 // flight per lane (six of 32 k or three of 64 k: the same bytes).
-template <int TN, int WAVES_M, int KSPLIT, int BK = NT_BK, int RING = NT_RING>
-__global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
+template <int TN, int WAVES_M, int KSPLIT, int BK = NT_BK, int RING = NT_RING, int PER_CU = 1>
+__global__ __launch_bounds__(NT_THREADS, PER_CU) void gemm_f32_nt_kernel(GemmArgs p) {
     static_assert(WAVES_M * KSPLIT * WAVE == NT_THREADS, "8 waves per workgroup");
     static_assert(RING % NT_STAGES == 0, "a tile's LDS buffer is its ring slot modulo the number of buffers");
     constexpr int BM = 16 * WAVES_M, BN = 16 * TN, NT_PITCH = BK + LDS_PAD;
@@ -140,8 +140,11 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
                                                      16 * (c * KSPLIT + ks) + 4 * lq);
     };
 
-    auto tile_step = [&](auto r_tag, auto pre_tag, auto prea_tag, auto wr_tag, auto nxt_tag, int kt) {
-        constexpr int r = decltype(r_tag)::value;
+    // (u: the step's place in the unrolled group; the ring slot is u % RING, and the operand set alternates with every chunk,
+    // which only repeats after RING steps when RING * NC is even: an odd ring of single-chunk tiles is unrolled twice over)
+    constexpr int UNROLL = (RING * NC) % 2 == 0 ? RING : 2 * RING;
+    auto tile_step = [&](auto u_tag, auto pre_tag, auto prea_tag, auto wr_tag, auto nxt_tag, int kt) {
+        constexpr int u = decltype(u_tag)::value, r = u % RING;
         constexpr bool PRE = decltype(pre_tag)::value, PRE_A = decltype(prea_tag)::value;
         constexpr bool WR = decltype(wr_tag)::value, NXT = decltype(nxt_tag)::value;
         // The step's six memory instructions are spread between its MFMAs: issued
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
         constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            constexpr int g0 = (r * NC) & 1;
+            constexpr int g0 = (u * NC) & 1;
             const int cur = (g0 + c) & 1;
             // fragments of the next chunk: same tile, or chunk 0 of tile kt + 1 (visible since the last barrier)
             if (c + 1 < NC) read_b(bf[cur ^ 1], r % NT_STAGES, c + 1);
@@ -204,7 +207,7 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     // The small-tile variants have registers to spare: fetch this lane's bias and residual
     // values now, so the epilogue does not wait for two more trips to memory (k-split
     // group 1 never needs them).
-    constexpr bool PREFETCH_EPI = KSPLIT == 2 && TN <= 4;
+    constexpr bool PREFETCH_EPI = KSPLIT == 2 && TN <= 4 && PER_CU < 3;   // (three workgroups per CU leave no registers for it)
     f32x4 pre_bias[PREFETCH_EPI ? TN : 1], pre_res[PREFETCH_EPI ? TN : 1];
     if constexpr (PREFETCH_EPI) {
         const int64_t pm = m0 + 16 * wm + li;
@@ -230,11 +233,11 @@ __global__ __launch_bounds__(NT_THREADS) void gemm_f32_nt_kernel(GemmArgs p) {
     // off but clamped to the last tile (they re-read data that is already in cache and
     // write LDS buffers nobody reads any more), so the step body stays branch-free
     // and the compiler's s_waitcnt counts stay exact from the first tile to the last.
-    for (int kt0 = 0; kt0 < ktiles; kt0 += RING) {
-        nt_static_for<RING>([&](auto r_tag) {
-            const int kt = kt0 + decltype(r_tag)::value;
+    for (int kt0 = 0; kt0 < ktiles; kt0 += UNROLL) {
+        nt_static_for<UNROLL>([&](auto u_tag) {
+            const int kt = kt0 + decltype(u_tag)::value;
             if (kt < ktiles)  // uniform; only the last group can be partial
-                tile_step(r_tag, std::true_type{}, std::true_type{}, std::true_type{}, std::true_type{}, kt);
+                tile_step(u_tag, std::true_type{}, std::true_type{}, std::true_type{}, std::true_type{}, kt);
         });
     }
 
@@ -323,7 +326,15 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     // 41.9 us against 44.8 us with 32-k tiles and 43.9 us with six 64-k tiles in flight; the wider
     // variants lose 1-2 % with 64-k tiles)
     const bool bk64 = p.K % 64 == 0 && (tune.gemm_nt_bk ? tune.gemm_nt_bk == 64 : true);
-    if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64, 3>), grid, block, 0, stream, p);
+    // ... and where K is short a lean form of it (32-k tiles, a three-deep ring, no early fetch of bias and residual: 69
+    // registers) of which three workgroups share a CU: all 768 tiles of 1024 x 2304 x 768 are resident at once (32.4 against
+    // 34.0 us), and a workgroup that has its CU to itself starts sooner with half the bytes in its first burst
+    // (1024 x 768 x 768: 13.1 against 13.6 us). With its 64 k of look-ahead it falls behind once the operands no longer sit
+    // in the L2 (1024 x 768 x 1536: 25.8 against 22.9 us; with three workgroups per CU it holds up to K = 1536).
+    // MI355X_GEMM_NT_PER_CU: 3 forces it, 2 forbids it.
+    const bool lean = tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : (p.K <= 1024 || (p.K <= 1536 && p.nwg > 2 * (int64_t)cus));
+    if (best == 0 && lean && tune.gemm_nt_bk == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 3>), grid, block, 0, stream, p);
+    else if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64, 3>), grid, block, 0, stream, p);
     else if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
