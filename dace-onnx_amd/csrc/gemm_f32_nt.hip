@@ -339,6 +339,12 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
     else if (best == 2) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
+    // the same for 128 x 48 tiles (80 registers): where all tiles are resident at once and K is short, 1024 x 3072 x 768 with
+    // Gelu takes 40.0 against 42.2 us; 4096 x 4096 x 1024 (3.6 rounds of 768 places) 246 against 262 us, but 2048 x 3072 x 768
+    // (1024 tiles on 768 places: the last third of a round runs one to a CU) 87.5 against 77.7 us, so only the first case
+    // is taken. MI355X_GEMM_NT_PER_CU=3 forces it here too.
+    else if (best == 4 && tune.gemm_nt_bk == 0 && (tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : (p.K <= 1024 && p.nwg <= 3 * (int64_t)cus)))
+        hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1, 32, 3, 2>), grid, block, 0, stream, p);
     else if (best == 4 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1, 64, 3>), grid, block, 0, stream, p);
     else if (best == 4) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((gemm_f32_nt_kernel<9, 4, 2>), grid, block, 0, stream, p);
