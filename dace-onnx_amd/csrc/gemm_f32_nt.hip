@@ -23,6 +23,7 @@
 //     visible since the barrier of tile t - 1); one barrier per tile.
 // MFMA operands are swapped as in gemm_f32.hip: a lane's accumulator registers
 // are four consecutive n of one row, stored as 16 bytes.
+#include <algorithm>
 #include "common.h"
 #include "gemm_tile.h"
 #include "gemm_args.h"
@@ -280,7 +281,15 @@ __global__ __launch_bounds__(NT_THREADS, PER_CU) void gemm_f32_nt_kernel(GemmArg
     MI355X_TRACE_STAMP(p, 3);
 }
 
-// The caller guarantees: 16-byte aligned operands, a_sk == b_sk == 1, every stride
+// 128 x 48 tiles: true where the deep-ring kernel (two workgroups per CU) fills its last round and the lean one (three
+// per CU) would leave most of its last round empty -- the one pattern in which the deep ring measured faster.
+static bool deep_ring_rounds_fit(int64_t nwg, int cus, int64_t K) {
+    const int64_t deep = 2 * (int64_t)cus, lean = 3 * (int64_t)cus;
+    if (nwg <= lean || nwg > 4 * deep || K > 2048 || (nwg > 2 * deep && K < 768)) return false;   // (2048 tiles at K = 512: 99 against 110 us)
+    const int64_t deep_empty = (deep - nwg % deep) % deep, lean_empty = (lean - nwg % lean) % lean;   // free places in the last round
+    return deep_empty * 8 <= deep && lean_empty * 10 >= 3 * lean;
+}
+
 // and N a multiple of 4. Additionally needed here: K a multiple of the 32-k tile.
 bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     if (p.K % NT_BK != 0 || p.K == 0) return false;
@@ -303,7 +312,9 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     const int force = tune.gemm_nt_bn, force_bm = tune.gemm_nt_bm;
     for (int c = 0; c < 5; ++c) {
         const int64_t nwg = p.batch * ceil_div(p.M, cands[c].bm) * ceil_div(p.N, cands[c].bn);
-        const double cost = (double)ceil_div(nwg, (int64_t)cus * cands[c].per_cu) * cands[c].per_cu * cands[c].bm * cands[c].bn * cands[c].weight;
+        double cost = (double)ceil_div(nwg, (int64_t)cus * cands[c].per_cu) * cands[c].per_cu * cands[c].bm * cands[c].bn * cands[c].weight;
+        // (128 x 48 also runs three to a CU, in its lean form, 5 % faster per tile at full occupancy)
+        if (c == 4) cost = std::min(cost, (double)ceil_div(nwg, (int64_t)cus * 3) * 3 * cands[c].bm * cands[c].bn * 0.74);
         if (force) {   // MI355X_GEMM_NT_BN picks the tile width, MI355X_GEMM_NT_BM the height where two candidates share a width
             if (force == cands[c].bn && (force_bm ? force_bm == cands[c].bm : cands[c].bm == 64 || cands[c].bn == 96)) { best = c; break; }
         } else if (cost < best_cost) {
@@ -318,7 +329,9 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     // an XCD holds cus / 8 tiles at a time (twice that for the candidates that run in pairs)
     const int64_t per_xcd = ceil_div(p.nwg, (int64_t)NUM_XCD);
     const int64_t per_batch = p.tiles_m * p.tiles_n;   // tiles are numbered batch entry by batch entry
-    p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, (int64_t)cands[best].per_cu * (cus / NUM_XCD), cands[best].bm, cands[best].bn, p.K * 4);
+    // (the lean 128 x 48 kernel, chosen below, runs three workgroups per CU)
+    const bool lean128 = best == 4 && tune.gemm_nt_bk == 0 && (tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : !deep_ring_rounds_fit(p.nwg, cus, p.K));
+    p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, (int64_t)(lean128 ? 3 : cands[best].per_cu) * (cus / NUM_XCD), cands[best].bm, cands[best].bn, p.K * 4);
     if (tune.gemm_group_m > 0) p.group_m = tune.gemm_group_m;
     const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
     // The smallest variant walks K in 64-k tiles with a three-deep ring where K allows: half the barriers per FLOP
@@ -339,11 +352,14 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
     else if (best == 2) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
-    // the same for 128 x 48 tiles (80 registers): where all tiles are resident at once and K is short, 1024 x 3072 x 768 with
-    // Gelu takes 40.0 against 42.2 us; 4096 x 4096 x 1024 (3.6 rounds of 768 places) 246 against 262 us, but 2048 x 3072 x 768
-    // (1024 tiles on 768 places: the last third of a round runs one to a CU) 87.5 against 77.7 us, so only the first case
-    // is taken. MI355X_GEMM_NT_PER_CU=3 forces it here too.
-    else if (best == 4 && tune.gemm_nt_bk == 0 && (tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : (p.K <= 1024 && p.nwg <= 3 * (int64_t)cus)))
+    // the same for 128 x 48 tiles (80 registers, three workgroups per CU): 1024 x 3072 x 768 with Gelu takes 40.0 against
+    // 42.2 us, 4096 x 4096 x 1024 246 against 262 us. Measured over 3072-wide outputs of 512 to 3328 tiles and K from 768
+    // to 4096 it wins by 5-7 % at K = 768, 3-4 % at 1536 and 1-2 % from 2048 on, with one exception: where the tiles fill
+    // whole rounds of two per CU but not of three (1024 tiles on 256 CUs: 88.0 against 78.3 us at K = 768, 160 against
+    // 144 us at 1536, 197 against 184 us at 2048, even from K = 3072 on; 2048 tiles: even at 768, 293 against 282 us at
+    // 1536) the leftover third of a round runs one or two workgroups to a CU, where the short ring cannot cover the
+    // latency. MI355X_GEMM_NT_PER_CU: 3 forces it, 2 forbids it.
+    else if (lean128)
         hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1, 32, 3, 2>), grid, block, 0, stream, p);
     else if (best == 4 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1, 64, 3>), grid, block, 0, stream, p);
     else if (best == 4) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 8, 1>), grid, block, 0, stream, p);

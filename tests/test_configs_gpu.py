@@ -309,6 +309,40 @@ def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
     assert rel_err(ref.cpu().numpy(), out.cpu().numpy()) < FP32_REL_TOL
 
 
+@pytest.mark.parametrize("M, N, K, epi", [(1100, 3076, 96, 5),     # 2 x 9 x 65 = 1170 tiles of 128 x 48: several rounds of three per CU, ragged in M and N
+                                          (1024, 3072, 64, 9),     # 1024 tiles: whole rounds of two per CU, the deep-ring kernel
+                                          (3000, 2308, 160, 1)])   # 2 x 24 x 49 = 2352 tiles
+def test_k_contiguous_gemm_several_rounds_of_workgroups(tuning, M, N, K, epi):
+    """The library's own choice between the deep-ring and the lean 128 x 48 kernel on problems of several rounds of
+    workgroups, against the same product with 64 x 48 tiles forced and against float64."""
+    lib = _lib.library()
+    rng = np.random.default_rng(M + N + K)
+    a = torch.from_numpy(rng.normal(size=(2, M, K)).astype(np.float32)).cuda()
+    w = torch.from_numpy(rng.normal(size=(N, K)).astype(np.float32)).cuda()
+    bias = torch.from_numpy(rng.normal(size=N).astype(np.float32)).cuda()
+    res = torch.from_numpy(rng.normal(size=(2, M, N)).astype(np.float32)).cuda()
+
+    def product():
+        out = torch.full((2, M, N), float("nan"), device="cuda")
+        _lib.check(lib.mi355x_gemm_f32(a.data_ptr(), w.data_ptr(), out.data_ptr(), bias.data_ptr(), res.data_ptr(), 1, 2, M, N, K,
+                                       _lib.i64_array([0, M * K, K, 1]), _lib.i64_array([0, 0, 1, K]), _lib.i64_array([0, M * N, N]),
+                                       _lib.i64_array([0, M * N, N]), 1.0, epi, _lib.current_stream()), "gemm")
+        return out
+
+    tuning()
+    chosen = product()
+    tuning(MI355X_GEMM_NT_BN=48, MI355X_GEMM_NT_PER_CU=2)
+    small_tiles = product()
+    ref = a.double() @ w.double().T + bias.double()
+    if epi & 4:
+        ref = torch.nn.functional.gelu(ref)
+    if epi & 8:
+        ref = ref + res.double()
+    assert rel_err(ref.cpu().numpy(), chosen.cpu().numpy()) < FP32_REL_TOL
+    # the same products in another order of summation (one chain against two k-split chains): fp32 rounding apart
+    torch.testing.assert_close(chosen, small_tiles, rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("variables", [{"MI355X_GEMM_CONFIG": c} for c in range(5)] + [{"MI355X_GEMM_NT_BK": 32},
                                                                                         {"MI355X_GEMM_NT_BK": 32, "MI355X_GEMM_NT_BN": 64},
                                                                                         {"MI355X_GEMM_GROUP_M": 1}, {"MI355X_GEMM_KSPLIT": 1},
