@@ -241,8 +241,13 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     if (cus <= 0) return set_error(MI355X_ERR_NOT_INITIALIZED, "gemm: no usable HIP device");
     // both operands contiguous along k (activations x pre-transposed weights, Q K^T):
     // the dedicated kernel reads every MFMA fragment with 16-byte accesses
+    // (not for stacks of small products over a short K -- the scores of an attention head, 96 x (128 x 128 x 64): the
+    // kernel's register ring is longer than their K, and 32 x 64 tiles of four waves fill the part better: 7.4 against
+    // 9.1 us, 128 x 128 x 128 9.9 against 11.0 us, 128 x 128 x 32 6.1 against 8.2 us)
     const Tuning tune = tuning();
-    if (a_kc && b_kc && vec && tune.gemm_config < 0) {
+    const bool small_stack = batch > 1 && M <= 128 && N <= 128 && K <= 128 &&   // (a forced variant of that kernel is taken all the same)
+                             tune.gemm_nt_bn == 0 && tune.gemm_nt_per_cu == 0 && tune.gemm_nt_bk == 0 && tune.gemm_ksplit != 1;
+    if (a_kc && b_kc && vec && tune.gemm_config < 0 && !small_stack) {
         // MI355X_GEMM_KSPLIT: 1 sends every such product to the kernel whose waves split K, 0 none
         if (tune.gemm_ksplit == 1 && launch_gemm_f32_ksplit(p, cus, static_cast<hipStream_t>(stream)))
             return check_launch("gemm_f32_ksplit_kernel");

@@ -346,7 +346,9 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     // in the L2 (1024 x 768 x 1536: 25.8 against 22.9 us; with three workgroups per CU it holds up to K = 1536).
     // MI355X_GEMM_NT_PER_CU: 3 forces it, 2 forbids it.
     const bool lean = tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : (p.K <= 1024 || (p.K <= 1536 && p.nwg > 2 * (int64_t)cus));
-    if (best == 0 && lean && tune.gemm_nt_bk == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 3>), grid, block, 0, stream, p);
+    // (a workgroup that has its CU to itself also has the registers to fetch its bias and residual values before the loop)
+    if (best == 0 && lean && tune.gemm_nt_bk == 0 && p.nwg <= cus && tune.gemm_nt_per_cu != 3) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 1>), grid, block, 0, stream, p);
+    else if (best == 0 && lean && tune.gemm_nt_bk == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 3>), grid, block, 0, stream, p);
     else if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64, 3>), grid, block, 0, stream, p);
     else if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
