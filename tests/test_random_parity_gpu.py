@@ -71,6 +71,42 @@ def test_random_gemm(seed):
     assert not failures, failures
 
 
+def test_random_gemm_many_tiles():
+    """Both operands k-contiguous, outputs of several hundred to several thousand tiles: the shapes on which the
+    library chooses between 64 x 48 and 128 x 48 tiles, between the deep and the lean register ring and between one,
+    two and three workgroups per CU, with extents that leave partial tiles and partial rounds of workgroups."""
+    lib, stream = _lib_and_stream()
+    rng, dev, failures = np.random.default_rng(7), "cuda", []
+    for case in range(24):
+        b1 = int(rng.choice([1, 1, 1, 2]))
+        M, N, K = int(rng.integers(500, 4600)), 4 * int(rng.integers(150, 1100)), 32 * int(rng.integers(1, 24))
+        if case % 6 == 0:   # whole rounds of two workgroups per CU: the pattern that keeps the deep ring
+            M, N, b1 = 128 * int(rng.choice([8, 16, 32])), 48 * 64, 1
+        A = torch.from_numpy(rng.normal(size=(1, b1, M, K)).astype(np.float32)).to(dev)
+        W = torch.from_numpy(rng.normal(size=(N, K)).astype(np.float32)).to(dev)
+        epi = int(rng.choice([0, 1, 5, 9]))
+        bias = torch.from_numpy(rng.normal(size=N).astype(np.float32)).to(dev)
+        res = torch.from_numpy(rng.normal(size=(1, b1, M, N)).astype(np.float32)).to(dev)
+        C = torch.full((1, b1, M, N), float("nan"), device=dev)
+        ref = A.double() @ W.double().T
+        if epi & _lib.EPI_BIAS:
+            ref = ref + bias.double()
+        if epi & _lib.EPI_GELU:
+            ref = torch.nn.functional.gelu(ref)
+        if epi & _lib.EPI_RESIDUAL:
+            ref = ref + res.double()
+        tag = f"gemm many tiles case {case}: b{b1} M{M} N{N} K{K} epi={epi}"
+        print(tag, flush=True)
+        st = lib.mi355x_gemm_f32(A.data_ptr(), W.data_ptr(), C.data_ptr(), bias.data_ptr(), res.data_ptr(), 1, b1, M, N, K,
+                                 _lib.i64_array([0, M * K, K, 1]), _lib.i64_array([0, 0, 1, K]), _lib.i64_array([0, M * N, N]),
+                                 _lib.i64_array([0, M * N, N]), 1.0, epi, stream())
+        torch.cuda.synchronize()
+        if st != 0 or torch.isnan(C).any().item() or _rel(C, ref) >= FP32_REL_TOL:
+            failures.append(tag)
+        del A, W, C, ref, res
+    assert not failures, failures
+
+
 @pytest.mark.parametrize("seed", [0, 1])
 def test_random_conv(seed):
     lib, stream = _lib_and_stream()
