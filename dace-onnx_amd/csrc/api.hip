@@ -61,6 +61,7 @@ static void parse_tuning(Tuning& t) {
     t.conv_gather_bn = env_int("MI355X_CONV_GATHER_BN", 0);
     t.conv_tail = env_int("MI355X_CONV_TAIL", -1);
     t.conv_static_taps = env_int("MI355X_CONV_STATIC_TAPS", 1);
+    t.conv_per_cu = env_int("MI355X_CONV_PER_CU", 0);
     t.mmi_generic = getenv("MI355X_MMI_GENERIC") != nullptr;
     t.mmi_wgs_per_cu = env_int("MI355X_MMI_WGS_PER_CU", 0);
     t.mmi_tile = env_int("MI355X_MMI_TILE", 0);

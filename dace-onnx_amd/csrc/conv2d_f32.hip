@@ -262,12 +262,16 @@ constexpr int cg_gcd(int a, int b) { return b == 0 ? a : cg_gcd(b, a % b); }
 // from its position's first pixel, plus one channel where j + rot wraps, with bit 31 set where that tap is
 // padding: the load of (i, e) takes register j (known at compile time) as its vector offset and the running
 // channel offset (a + 32 window + n) H W 4, kept on the scalar unit, as its scalar offset.
-template <int TN, int TAPS = 0>
+// LEAN: a three-deep register ring and one set of X operands instead of six and two (73 registers instead of 122), so
+// that three workgroups share a CU. The X operands of the next step are read from LDS into the registers of a pair of
+// position tiles as soon as the pair's MFMAs of this step have been issued.
+template <int TN, int TAPS = 0, bool LEAN = false>
 __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_t m0, int64_t p0, float* lds, uint32_t* lds_tap) {
-    constexpr int BN = 16 * TN, BK = CG_BK, RING = CG_RING, PITCH = CG_PITCH;
+    constexpr int BN = 16 * TN, BK = CG_BK, RING = LEAN ? CG_STAGES : CG_RING, PITCH = CG_PITCH;
     constexpr bool STATIC_TAPS = TAPS > 0;
     constexpr int WIN = STATIC_TAPS ? TAPS / cg_gcd(BK, TAPS ? TAPS : 1) : 1;        // steps per window
-    constexpr int UNROLL = RING * WIN / cg_gcd(RING, WIN);                           // slot and window position both fixed
+    constexpr int UNROLL1 = RING * WIN / cg_gcd(RING, WIN);                          // slot and window position both fixed
+    constexpr int UNROLL = UNROLL1 % 2 == 0 ? UNROLL1 : 2 * UNROLL1;                 // ... and the operand set (step parity)
     constexpr int NTAP = STATIC_TAPS ? TAPS : 1;
     constexpr int UNITS = BN * (BK / 4);                 // (position, k-quad) units of one tile
     // whole waves of loader units share their k-quad (read once, on the scalar unit); a narrow slice has four
@@ -371,7 +375,7 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     const int last_tile = ktiles - 1;
     f32x4 ra[RING];            // W operand of tile t in slot t % RING
     f32x4 rb[RING][B_PER_T];   // gathered pixels of tile t in slot t % RING
-    f32x4 bf[2][TN];           // X operands of tile t in set t % 2
+    f32x4 bf[LEAN ? 1 : 2][TN];   // X operands of tile t in set t % 2 (lean: one set, refilled pair by pair)
 
     auto load_a = [&](f32x4& dst, int kt) __attribute__((always_inline)) {
         dst = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, (int)a_off, (kt < last_tile ? kt : last_tile) * (BK * 4), 0));
@@ -433,10 +437,42 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
 
     auto tile_step = [&](auto u_tag, int kt) __attribute__((always_inline)) {
         constexpr int r = decltype(u_tag)::value % RING;
-        constexpr int cur = r & 1;  // RING is even: tile parity == slot parity
+        constexpr int cur = LEAN ? 0 : (decltype(u_tag)::value & 1);  // UNROLL is even: tile parity == step parity
         load_b(rb[r], kt + RING, std::integral_constant<int, (decltype(u_tag)::value + RING) % WIN>{});   // slot r went to LDS two steps ago
         load_a(ra[(r + RING - 1) % RING], kt + RING - 1);   // operand consumed in the previous step
         store_b(rb[(r + 2) % RING], (r + 2) % CG_STAGES);   // tile kt + 2
+        constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
+        if constexpr (LEAN) {
+            // position tiles in pairs (two independent accumulators alternate); the pair's operands of tile kt + 1,
+            // visible since the last barrier, replace this step's once its MFMAs have been issued
+#pragma unroll
+            for (int j0 = 0; j0 < TN; j0 += 2) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int j = j0; j < j0 + 2 && j < TN; ++j)
+                        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[0][j][s], ra[r][s], acc[j], 0, 0, 0);
+#pragma unroll
+                for (int j = j0; j < j0 + 2 && j < TN; ++j)
+                    bf[0][j] = *reinterpret_cast<const f32x4*>(lds + ((r + 1) % CG_STAGES) * STAGE + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
+            }
+            if constexpr (UNIFORM_KQ && TN == 4) {
+                __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
+                if constexpr (!STATIC_TAPS) __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
+#pragma unroll
+                for (int v = 0; v < 4 * B_PER_T + 1; ++v) {
+                    __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(VMEM_RD, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(MFMA, 8 - 1 - (4 * B_PER_T + 1), 0);
+                __builtin_amdgcn_sched_group_barrier(DS_RD, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(MFMA, 8, 0);
+                __builtin_amdgcn_sched_group_barrier(DS_RD, 2, 0);
+            }
+            __syncthreads();
+            return;
+        }
         read_b(bf[cur ^ 1], (r + 1) % CG_STAGES);           // tile kt + 1, visible since the last barrier
 #pragma unroll
         for (int s = 0; s < 4; ++s)
@@ -446,7 +482,6 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         // Issue order: LDS traffic first (it must have completed at the barrier), then the
         // gather loads, each memory instruction between MFMAs so that it never queues
         // behind the other waves' requests while the matrix pipe idles.
-        constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
         if constexpr (UNIFORM_KQ) {
         __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
         __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
@@ -465,7 +500,8 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         }
         __syncthreads();
     };
-    static_assert(RING % 2 == 0 && RING % CG_STAGES == 0, "slot index fixes operand set and LDS buffer");
+    static_assert(UNROLL % 2 == 0 && RING % CG_STAGES == 0, "step index fixes operand set, slot index the LDS buffer");
+    static_assert(!LEAN || 4 * B_PER_T + 2 <= 8, "the lean step's memory instructions fit between the first pair's MFMAs");
 
 #pragma unroll
     for (int r = 0; r < RING; ++r) load_a(ra[r], r);  // tiles beyond the last are clamped: no branch
@@ -552,8 +588,8 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
 }
 
 // TN: the whole tiles; workgroups past p.full_tiles take 16-position slices (TN = 1)
-template <int TN, int TAPS>
-__global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs p) {
+template <int TN, int TAPS, bool LEAN = false>
+__global__ __launch_bounds__(CG_THREADS, LEAN ? 3 : 1) void conv2d_f32_gather_kernel(ConvArgs p) {
     __shared__ __attribute__((aligned(16))) float lds[cg_lds_floats(TN)];
     // tap table: for every k = (c, r, s) the element offset of that tap relative to a
     // position's top-left input pixel (low 27 bits) and the tap index r * KW + s (high 5 bits)
@@ -562,10 +598,10 @@ __global__ __launch_bounds__(CG_THREADS) void conv2d_f32_gather_kernel(ConvArgs 
         const int64_t logical = xcd_remap(blockIdx.x, p.full_tiles);
         int64_t tm, tn;
         tile_coords(logical, p.tiles_m, p.tiles_p, p.group_m, tm, tn);
-        conv2d_f32_gather_tile<TN, TAPS>(p, tm * CG_BM, tn * (16 * TN), lds, lds_tap);
+        conv2d_f32_gather_tile<TN, TAPS, LEAN>(p, tm * CG_BM, tn * (16 * TN), lds, lds_tap);
     } else {
         const uint32_t q = blockIdx.x - (uint32_t)p.full_tiles, tiles_m = (uint32_t)p.tiles_m;
-        conv2d_f32_gather_tile<1>(p, (int64_t)(q % tiles_m) * CG_BM, p.p_full + 16 * (int64_t)(q / tiles_m), lds, lds_tap);
+        conv2d_f32_gather_tile<1, 0, LEAN>(p, (int64_t)(q % tiles_m) * CG_BM, p.p_full + 16 * (int64_t)(q / tiles_m), lds, lds_tap);
     }
 }
 
@@ -660,14 +696,19 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
     if (K % CG_BK == 0 && K <= CG_MAX_K && KH * KW <= 32 && M * K < ((int64_t)1 << 29) && C * H * Wd < ((int64_t)1 << 27) &&
         N * C * H * Wd + pads[0] * Wd + pads[1] + H * Wd < ((int64_t)1 << 29) && al16(W) && tune.conv_config < 0) {
         p.x_bytes = (int)(N * C * H * Wd * 4);
-        // 64 x 64 tiles (two workgroups share a CU) or 64 x 128 (one per CU): both run a full CU
-        // at the same rate, so the choice is the number of rounds times the tile width; ties go
-        // to the narrow tile, whose last, partly filled round is shorter
-        auto cost = [&](int bn, int wgs_per_cu) {
+        // 64 x 64 tiles (three workgroups share a CU) or 64 x 128 (one per CU). Time goes with the tiles a CU has
+        // to run times their width; the wide tile, alone on its CU, pays its first loads and last stores in the open
+        // (32 x 64 x 56 x 56 -> 64: 101.5 us as 784 wide tiles, 73.2 us as 1568 narrow ones two to a CU), hence its factor.
+        auto cost = [&](int bn, double factor) {
             const int64_t tiles = ceil_div(M, (int64_t)CG_BM) * ceil_div(P, (int64_t)bn);
-            return ceil_div(tiles, (int64_t)cus * wgs_per_cu) * bn * wgs_per_cu;
+            return (double)ceil_div(tiles, (int64_t)cus) * bn * factor;
         };
-        const bool wide = tune.conv_gather_bn ? tune.conv_gather_bn == 128 : cost(128, 1) < cost(64, 2);
+        // The narrow tile runs as the lean kernel, three workgroups per CU (MI355X_CONV_PER_CU=2: the six-deep ring, two
+        // per CU): 32 x 64 x 56 x 56 -> 64, 3 x 3, takes 67.4 against 73.2 us, 16 x 256 x 28 x 28 -> 256 129.5 against
+        // 141.6 us, 16 x 64 x 28 x 28 -> 256 37.9 against 45.3 us, 1 x 1 over 32 x 64 x 56 x 56 -> 256 62.9 against 83.6 us;
+        // bit-equal results (each accumulator sees the same MFMAs in the same order).
+        const int per_cu = tune.conv_per_cu == 2 ? 2 : 3;
+        const bool wide = tune.conv_gather_bn ? tune.conv_gather_bn == 128 : cost(128, 1.3) < cost(64, 1.0);
         const int bn = wide ? 128 : 64;
         p.tiles_m = ceil_div(M, (int64_t)CG_BM);
         p.tiles_p = ceil_div(P, (int64_t)bn);
@@ -675,11 +716,12 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
         p.p_full = p.tiles_p * bn;
         int64_t slices = 0;
         // Narrow tiles in more than one round of workgroups, the last round less than half full (configuration 4:
-        // 1568 tiles on 512 places): the tiles of that round run as 16-position slices, four times as many
+        // 1568 tiles on 768 places): the tiles of that round run as 16-position slices, four times as many
         // workgroups of a quarter of the work each, so the places that would idle through a whole tile time
         // share its work.
+        const bool lean = !wide && per_cu == 3;
         if (!wide && tune.conv_tail != 0) {
-            const int64_t places = (int64_t)cus * 2, rem = p.full_tiles % places;
+            const int64_t places = (int64_t)cus * (lean ? 3 : 2), rem = p.full_tiles % places;
             const int64_t tail_p = tune.conv_tail > 0 ? tune.conv_tail : rem / p.tiles_m;
             const bool wanted = tune.conv_tail > 0 || (p.full_tiles > places && rem > 0 && rem < places / 2);
             if (wanted && tail_p > 0 && tail_p < p.tiles_p) {
@@ -698,6 +740,10 @@ extern "C" int mi355x_conv2d_res_f32(const float* X, const float* W, const float
             if (taps == 9) hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 9>), g, b, 0, st, p);
             else if (taps == 1) hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 1>), g, b, 0, st, p);
             else hipLaunchKernelGGL((conv2d_f32_gather_kernel<8, 0>), g, b, 0, st, p);
+        } else if (lean) {
+            if (taps == 9) hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 9, true>), g, b, 0, st, p);
+            else if (taps == 1) hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 1, true>), g, b, 0, st, p);
+            else hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 0, true>), g, b, 0, st, p);
         } else {
             if (taps == 9) hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 9>), g, b, 0, st, p);
             else if (taps == 1) hipLaunchKernelGGL((conv2d_f32_gather_kernel<4, 1>), g, b, 0, st, p);

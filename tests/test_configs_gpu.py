@@ -181,7 +181,7 @@ def test_config3_hip_graph_replays_match_eager(bert_case):
 
 
 # ----------------------------------------------------------------------------- config 4: ResNet Conv + Relu
-def test_config4_conv_relu_full_size(c_oracle):
+def test_config4_conv_relu_full_size(c_oracle, tuning):
     rng = np.random.default_rng(4)
     X = rng.normal(size=(32, 64, 56, 56)).astype(np.float32)
     W = (rng.normal(size=(64, 64, 3, 3)) * np.sqrt(2.0 / 576)).astype(np.float32)
@@ -205,6 +205,11 @@ def test_config4_conv_relu_full_size(c_oracle):
     donnx.ONNXConv(X=(2 * X).astype(np.float32), W=W, Y=Y2, pads=[1, 1, 1, 1])
     assert rel_err(2 * Y1, Y2) < 1e-6
     assert np.array_equal(np.maximum(Y1, 0), Y)
+    # the six-deep register ring (two workgroups per CU) in place of the lean kernel the library takes: same bits
+    tuning(MI355X_CONV_PER_CU=2)
+    Y3 = np.zeros_like(Y)
+    donnx.ONNXConv(X=X, W=W, Y=Y3, pads=[1, 1, 1, 1])
+    assert np.array_equal(Y1, Y3)
 
 
 # ----------------------------------------------------------------------------- config 5: MatMulInteger
@@ -617,7 +622,8 @@ def test_conv_residual_epilogue(shape, wshape, pads, strides, epi):
     ((2, 64, 16, 16), (80, 64, 3, 3), 7),      # two tiles of output channels (the second partly filled), 1 whole tile per row of tiles
     ((1, 32, 9, 9), (16, 32, 3, 3), 1)])       # 81 positions, odd: scalar stores in the slices
 @pytest.mark.parametrize("epi", [0, _lib.EPI_BIAS | _lib.EPI_RELU, _lib.EPI_BIAS | _lib.EPI_RESIDUAL | _lib.EPI_RELU_AFTER])
-def test_conv_last_round_as_slices(tuning, shape, wshape, tail, epi):
+@pytest.mark.parametrize("per_cu", [None, 2])   # the lean kernel the library takes (three workgroups per CU), the six-deep ring
+def test_conv_last_round_as_slices(tuning, shape, wshape, tail, epi, per_cu):
     """The convolution's last round of tiles run as 16-position slices (the library chooses that by the number of
     tiles and CUs; here it is forced on small problems through MI355X_CONV_TAIL = number of position tiles to slice)."""
     rng = np.random.default_rng(31 + tail)
@@ -637,7 +643,7 @@ def test_conv_last_round_as_slices(tuning, shape, wshape, tail, epi):
                       torch.cuda.current_stream().cuda_stream]
     results = []
     for setting in (str(tail), "0"):
-        tuning(MI355X_CONV_TAIL=setting)
+        tuning(MI355X_CONV_TAIL=setting, MI355X_CONV_PER_CU=per_cu)
         y = torch.full(pre.shape, float("nan"), device="cuda")
         assert lib.mi355x_conv2d_res_f32(*args(y)) == 0, lib.mi355x_last_error()
         torch.cuda.synchronize()
@@ -658,7 +664,8 @@ def test_conv_last_round_as_slices(tuning, shape, wshape, tail, epi):
 def test_conv_taps_known_at_compile_time(tuning, shape, wshape, strides, pads, dilations, gather_bn):
     """3 x 3 and 1 x 1 filters over a multiple of 32 channels take a gather whose tap offsets are compile-time
     register choices plus a scalar channel offset; MI355X_CONV_STATIC_TAPS=0 sends the same call through the tap
-    table. Both add up the same products in the same order."""
+    table, MI355X_CONV_PER_CU=2 through the six-deep register ring instead of the lean kernel (64-position tiles
+    only). All add up the same products in the same order."""
     rng = np.random.default_rng(77 + shape[1])
     x = rng.normal(size=shape).astype(np.float32)
     w = (rng.normal(size=wshape) / np.sqrt(np.prod(wshape[1:]))).astype(np.float32)
@@ -667,8 +674,8 @@ def test_conv_taps_known_at_compile_time(tuning, shape, wshape, strides, pads, d
     tx, tw, tb = (torch.from_numpy(a).cuda() for a in (x, w, b))
     lib = _lib.library()
     results = []
-    for setting in ("1", "0"):
-        tuning(MI355X_CONV_GATHER_BN=gather_bn, MI355X_CONV_STATIC_TAPS=setting)
+    for setting, per_cu in (("1", None), ("0", None), ("1", 2), ("0", 2)):
+        tuning(MI355X_CONV_GATHER_BN=gather_bn, MI355X_CONV_STATIC_TAPS=setting, MI355X_CONV_PER_CU=per_cu)
         y = torch.full(expected.shape, float("nan"), device="cuda")
         status = lib.mi355x_conv2d_f32(tx.data_ptr(), tw.data_ptr(), tb.data_ptr(), y.data_ptr(), *shape, wshape[0], wshape[2], wshape[3],
                                        _lib.i64_array(pads), _lib.i64_array(strides), _lib.i64_array(dilations),
@@ -677,7 +684,8 @@ def test_conv_taps_known_at_compile_time(tuning, shape, wshape, strides, pads, d
         torch.cuda.synchronize()
         results.append(y.cpu().numpy())
     assert rel_err(expected, results[0]) < FP32_REL_TOL
-    assert np.array_equal(results[0], results[1])
+    for other in results[1:]:
+        assert np.array_equal(results[0], other)
 
 
 def test_tasklet_fusion_programs_values():
