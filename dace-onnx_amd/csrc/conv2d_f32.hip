@@ -262,9 +262,9 @@ constexpr int cg_gcd(int a, int b) { return b == 0 ? a : cg_gcd(b, a % b); }
 // from its position's first pixel, plus one channel where j + rot wraps, with bit 31 set where that tap is
 // padding: the load of (i, e) takes register j (known at compile time) as its vector offset and the running
 // channel offset (a + 32 window + n) H W 4, kept on the scalar unit, as its scalar offset.
-// LEAN: a three-deep register ring and one set of X operands instead of six and two (73 registers instead of 122), so
-// that three workgroups share a CU. The X operands of the next step are read from LDS into the registers of a pair of
-// position tiles as soon as the pair's MFMAs of this step have been issued.
+// LEAN: a three-deep register ring and one set of X operands instead of six and two (78 registers instead of 122), so
+// that three workgroups share a CU. The X operands of half the position tiles are read from LDS under the MFMAs of the
+// other half.
 template <int TN, int TAPS = 0, bool LEAN = false>
 __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_t m0, int64_t p0, float* lds, uint32_t* lds_tap) {
     constexpr int BN = 16 * TN, BK = CG_BK, RING = LEAN ? CG_STAGES : CG_RING, PITCH = CG_PITCH;
@@ -443,20 +443,28 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
         store_b(rb[(r + 2) % RING], (r + 2) % CG_STAGES);   // tile kt + 2
         constexpr int MFMA = 0x008, VMEM_RD = 0x020, DS_RD = 0x100, DS_WR = 0x200;
         if constexpr (LEAN) {
-            // position tiles in pairs (two independent accumulators alternate); the pair's operands of tile kt + 1,
-            // visible since the last barrier, replace this step's once its MFMAs have been issued
+            // Position tiles in two halves. The step starts with the reads of the second half's operands of this tile
+            // (they land under the first half's MFMAs); the first half's operands of tile kt + 1, visible since the last
+            // barrier, replace this step's once its MFMAs have been issued: no LDS read is outstanding at the barrier.
+            constexpr int H = (TN + 1) / 2;
+            auto read_half = [&](int from, int to, int stage) __attribute__((always_inline)) {
 #pragma unroll
-            for (int j0 = 0; j0 < TN; j0 += 2) {
+                for (int j = from; j < to; ++j)
+                    bf[0][j] = *reinterpret_cast<const f32x4*>(lds + stage * STAGE + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
+            };
+            auto mfma_half = [&](int from, int to) __attribute__((always_inline)) {
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
 #pragma unroll
-                    for (int j = j0; j < j0 + 2 && j < TN; ++j)
+                    for (int j = from; j < to; ++j)
                         acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf[0][j][s], ra[r][s], acc[j], 0, 0, 0);
-#pragma unroll
-                for (int j = j0; j < j0 + 2 && j < TN; ++j)
-                    bf[0][j] = *reinterpret_cast<const f32x4*>(lds + ((r + 1) % CG_STAGES) * STAGE + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
-            }
+            };
+            read_half(H, TN, r % CG_STAGES);
+            mfma_half(0, H);
+            read_half(0, H, (r + 1) % CG_STAGES);
+            mfma_half(H, TN);
             if constexpr (UNIFORM_KQ && TN == 4) {
+                __builtin_amdgcn_sched_group_barrier(DS_RD, 2, 0);
                 __builtin_amdgcn_sched_group_barrier(MFMA, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(DS_WR, B_PER_T, 0);
                 if constexpr (!STATIC_TAPS) __builtin_amdgcn_sched_group_barrier(DS_RD, B_PER_T, 0);  // tap table
@@ -468,7 +476,6 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
                 __builtin_amdgcn_sched_group_barrier(MFMA, 8 - 1 - (4 * B_PER_T + 1), 0);
                 __builtin_amdgcn_sched_group_barrier(DS_RD, 2, 0);
                 __builtin_amdgcn_sched_group_barrier(MFMA, 8, 0);
-                __builtin_amdgcn_sched_group_barrier(DS_RD, 2, 0);
             }
             __syncthreads();
             return;
@@ -516,7 +523,12 @@ __device__ __forceinline__ void conv2d_f32_gather_tile(const ConvArgs& p, int64_
     store_b(rb[1], 1);
     MI355X_TRACE_STAMP(p, 7);
     __syncthreads();
-    read_b(bf[0], 0);
+    if constexpr (LEAN) {   // (the second half of tile 0 is read by step 0 itself)
+#pragma unroll
+        for (int j = 0; j < (TN + 1) / 2; ++j) bf[0][j] = *reinterpret_cast<const f32x4*>(lds + (16 * j + li) * PITCH + 16 * ks + 4 * lq);
+    } else {
+        read_b(bf[0], 0);
+    }
 
     // One code path for every tile: near the end of K the look-aheads are clamped to the
     // last tile, not switched off, so the step body stays branch-free.
