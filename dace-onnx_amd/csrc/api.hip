@@ -54,6 +54,7 @@ static void parse_tuning(Tuning& t) {
     t.gemm_nt_bk = env_int("MI355X_GEMM_NT_BK", 0);
     t.gemm_nt_bm = env_int("MI355X_GEMM_NT_BM", 0);
     t.gemm_nt_per_cu = env_int("MI355X_GEMM_NT_PER_CU", 0);
+    t.gemm_nt_waves = env_int("MI355X_GEMM_NT_WAVES", 0);
     t.gemm_group_m = env_int("MI355X_GEMM_GROUP_M", 0);
     t.gemm_ksplit = env_int("MI355X_GEMM_KSPLIT", -1);
     c = getenv("MI355X_CONV_CONFIG");

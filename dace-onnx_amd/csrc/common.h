@@ -24,7 +24,7 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Kernel-variant overrides from the MI355X_* environment variables (0 / -1 / false: not set), parsed once
 // and again on mi355x_reload_tuning(); CU count of the current device, asked of the runtime once per device.
 struct Tuning {
-    int gemm_config = -1, gemm_nt_bn = 0, gemm_nt_bm = 0, gemm_nt_bk = 0, gemm_nt_per_cu = 0, gemm_group_m = 0, gemm_ksplit = -1;
+    int gemm_config = -1, gemm_nt_bn = 0, gemm_nt_bm = 0, gemm_nt_bk = 0, gemm_nt_per_cu = 0, gemm_nt_waves = 0, gemm_group_m = 0, gemm_ksplit = -1;
     int conv_config = -1, conv_gather_bn = 0, conv_tail = -1, conv_static_taps = 1, conv_per_cu = 0;
     bool mmi_generic = false;
     int mmi_wgs_per_cu = 0, mmi_tile = 0;

@@ -246,7 +246,7 @@ extern "C" int mi355x_gemm_f32(const float* A, const float* B, float* C, const f
     // 9.1 us, 128 x 128 x 128 9.9 against 11.0 us, 128 x 128 x 32 6.1 against 8.2 us)
     const Tuning tune = tuning();
     const bool small_stack = batch > 1 && M <= 128 && N <= 128 && K <= 128 &&   // (a forced variant of that kernel is taken all the same)
-                             tune.gemm_nt_bn == 0 && tune.gemm_nt_per_cu == 0 && tune.gemm_nt_bk == 0 && tune.gemm_ksplit != 1;
+                             tune.gemm_nt_bn == 0 && tune.gemm_nt_per_cu == 0 && tune.gemm_nt_bk == 0 && tune.gemm_nt_waves == 0 && tune.gemm_ksplit != 1;
     if (a_kc && b_kc && vec && tune.gemm_config < 0 && !small_stack) {
         // MI355X_GEMM_KSPLIT: 1 sends every such product to the kernel whose waves split K, 0 none
         if (tune.gemm_ksplit == 1 && launch_gemm_f32_ksplit(p, cus, static_cast<hipStream_t>(stream)))

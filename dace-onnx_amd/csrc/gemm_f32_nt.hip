@@ -52,16 +52,17 @@ constexpr int NT_BK = 32, NT_THREADS = 512, NT_RING = 6, NT_STAGES = 3;
 // BK: k extent of a tile (32, or 64 where registers allow: half as many barriers per FLOP); RING: k-tiles in
 // flight per lane (six of 32 k or three of 64 k: the same bytes).
 template <int TN, int WAVES_M, int KSPLIT, int BK = NT_BK, int RING = NT_RING, int PER_CU = 1>
-__global__ __launch_bounds__(NT_THREADS, PER_CU) void gemm_f32_nt_kernel(GemmArgs p) {
-    static_assert(WAVES_M * KSPLIT * WAVE == NT_THREADS, "8 waves per workgroup");
+__global__ __launch_bounds__(WAVES_M * KSPLIT * WAVE, PER_CU) void gemm_f32_nt_kernel(GemmArgs p) {
+    constexpr int THREADS = WAVES_M * KSPLIT * WAVE;   // 8 waves, or 16 (4 wave rows x 4 k-split groups)
+    static_assert(THREADS == NT_THREADS || THREADS == 2 * NT_THREADS, "8 or 16 waves per workgroup");
     static_assert(RING % NT_STAGES == 0, "a tile's LDS buffer is its ring slot modulo the number of buffers");
     constexpr int BM = 16 * WAVES_M, BN = 16 * TN, NT_PITCH = BK + LDS_PAD;
     constexpr int NC = (BK / 16) / KSPLIT;  // 16-k chunks of a tile this wave multiplies
     constexpr int B_VECS = BN * (BK / 4);                       // 16-byte vectors of one B tile
-    constexpr int B_PER_T = (B_VECS + NT_THREADS - 1) / NT_THREADS;
-    constexpr int B_ROWS = B_PER_T * NT_THREADS / (BK / 4);     // rows incl. the ones only written as padding
+    constexpr int B_PER_T = (B_VECS + THREADS - 1) / THREADS;
+    constexpr int B_ROWS = B_PER_T * THREADS / (BK / 4);     // rows incl. the ones only written as padding
     constexpr int STAGE = B_ROWS * NT_PITCH;                    // floats per LDS buffer
-    constexpr int RED = (KSPLIT - 1) * BM * BN;                 // partial sums of k-split group 1
+    constexpr int RED = (KSPLIT - 1) * BM * BN;                 // partial sums of the k-split groups after the first
     constexpr int LDS_FLOATS = NT_STAGES * STAGE > RED ? NT_STAGES * STAGE : RED;
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
 
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(NT_THREADS, PER_CU) void gemm_f32_nt_kernel(GemmArg
     int b_lds[B_PER_T];
 #pragma unroll
     for (int it = 0; it < B_PER_T; ++it) {
-        const int idx = tid + it * NT_THREADS;
+        const int idx = tid + it * THREADS;
         const int row = idx / (BK / 4), c4 = idx % (BK / 4);
         int64_t bn = n0 + row;
         bn = bn < p.N ? bn : p.N - 1;
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(NT_THREADS, PER_CU) void gemm_f32_nt_kernel(GemmArg
     // The small-tile variants have registers to spare: fetch this lane's bias and residual
     // values now, so the epilogue does not wait for two more trips to memory (k-split
     // group 1 never needs them).
-    constexpr bool PREFETCH_EPI = KSPLIT == 2 && TN <= 4 && PER_CU < 3;   // (three workgroups per CU leave no registers for it)
+    constexpr bool PREFETCH_EPI = KSPLIT >= 2 && TN <= 4 && PER_CU < 3;   // (three workgroups per CU leave no registers for it)
     f32x4 pre_bias[PREFETCH_EPI ? TN : 1], pre_res[PREFETCH_EPI ? TN : 1];
     if constexpr (PREFETCH_EPI) {
         const int64_t pm = m0 + 16 * wm + li;
@@ -244,17 +245,19 @@ __global__ __launch_bounds__(NT_THREADS, PER_CU) void gemm_f32_nt_kernel(GemmArg
 
     MI355X_TRACE_STAMP(p, 2);
     MI355X_TRACE_CYCLES(p, 13);
-    // k-split group 1 hands its partial sums to group 0 through LDS
-    if constexpr (KSPLIT == 2) {
+    // the k-split groups after the first hand their partial sums to group 0 through LDS (added in the order of the groups)
+    if constexpr (KSPLIT >= 2) {
         f32x4* red = reinterpret_cast<f32x4*>(lds);
-        if (ks == 1) {
+        if (ks >= 1) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) red[(wm * TN + j) * WAVE + lane] = acc[j];
+            for (int j = 0; j < TN; ++j) red[(((ks - 1) * WAVES_M + wm) * TN + j) * WAVE + lane] = acc[j];
         }
         __syncthreads();
-        if (ks == 1) return;
+        if (ks >= 1) return;
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[j] += red[(wm * TN + j) * WAVE + lane];
+        for (int g = 1; g < KSPLIT; ++g)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[j] += red[(((g - 1) * WAVES_M + wm) * TN + j) * WAVE + lane];
     }
 
     // epilogue: acc[j][r] = C[m0 + 16*wm + li][n0 + 16*j + 4*lq + r]
@@ -333,7 +336,7 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     const bool lean128 = best == 4 && tune.gemm_nt_bk == 0 && (tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : !deep_ring_rounds_fit(p.nwg, cus, p.K));
     p.group_m = choose_group_m(p.tiles_m, per_xcd < per_batch ? per_xcd : per_batch, (int64_t)(lean128 ? 3 : cands[best].per_cu) * (cus / NUM_XCD), cands[best].bm, cands[best].bn, p.K * 4);
     if (tune.gemm_group_m > 0) p.group_m = tune.gemm_group_m;
-    const dim3 grid((unsigned)p.nwg), block(NT_THREADS);
+    const dim3 grid((unsigned)p.nwg), block(NT_THREADS), block16(2 * NT_THREADS);
     // The smallest variant walks K in 64-k tiles with a three-deep ring where K allows: half the barriers per FLOP
     // and the same bytes in flight as six 32-k tiles (1024 x 768 x 768: 14.0 us against 14.7 us, 1024 x 768 x 3072:
     // 41.9 us against 44.8 us with 32-k tiles and 43.9 us with six 64-k tiles in flight; the wider
@@ -347,7 +350,15 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     // MI355X_GEMM_NT_PER_CU: 3 forces it, 2 forbids it.
     const bool lean = tune.gemm_nt_per_cu ? tune.gemm_nt_per_cu == 3 : (p.K <= 1024 || (p.K <= 1536 && p.nwg > 2 * (int64_t)cus));
     // (a workgroup that has its CU to itself also has the registers to fetch its bias and residual values before the loop)
-    if (best == 0 && lean && tune.gemm_nt_bk == 0 && p.nwg <= cus && tune.gemm_nt_per_cu != 3) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 1>), grid, block, 0, stream, p);
+    // A workgroup that has its CU to itself over a long K runs as 16 waves, 4 wave rows x 4 k-split groups on 64-k tiles
+    // (four waves per SIMD cover each other's barrier waits; 104 registers): 1024 x 768 x 3072 38.0 against 39.8 us,
+    // 512 x 768 x 3072 37.2 against 39.5 us, 1024 x 768 x 1536 21.6 against 22.5 us; at K = 768 the lean kernel wins
+    // (12.4 against 13.0 us), and with more than one tile per CU eight waves do (1024 x 2304 x 768: 31.0 against 35.8 us).
+    // 128-k tiles or six 64-k tiles in flight (128 registers) are slower everywhere. MI355X_GEMM_NT_WAVES: 16 forces it, 8 forbids it.
+    const bool waves16 = best == 0 && p.K % 64 == 0 && tune.gemm_nt_bk == 0 &&
+                         (tune.gemm_nt_waves ? tune.gemm_nt_waves == 16 : (p.nwg <= cus && p.K >= 1280 && tune.gemm_nt_per_cu == 0));
+    if (waves16) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 4, 64, 3, 1>), grid, block16, 0, stream, p);
+    else if (best == 0 && lean && tune.gemm_nt_bk == 0 && p.nwg <= cus && tune.gemm_nt_per_cu != 3) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 1>), grid, block, 0, stream, p);
     else if (best == 0 && lean && tune.gemm_nt_bk == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 32, 3, 3>), grid, block, 0, stream, p);
     else if (best == 0 && bk64) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2, 64, 3>), grid, block, 0, stream, p);
     else if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);

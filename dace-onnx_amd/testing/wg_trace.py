@@ -81,16 +81,21 @@ def _workloads(lib, torch):
             "out_ksplit": ksplit(gemm(1024, 768, 768, 9)), "ffn2_ksplit": ksplit(gemm(1024, 768, 3072, 9))}
 
 
-def trace(name: str, warm_launches: int = 500, max_workgroups: int = 65536):
-    """Runs workload ``name`` once with stamps (after ``warm_launches`` without) and returns the stamps in
+def trace(name: str, warm_seconds: float = 0.3, max_workgroups: int = 65536):
+    """Runs workload ``name`` once with stamps (after ``warm_seconds`` of launches without) and returns the stamps in
     microseconds relative to the first workgroup's start, ``[workgroups, 4]``, and the CU key of each workgroup."""
+    import time
     import torch
     lib = load_trace_library()
     launch, keep = _workloads(lib, torch)[name]()
     os.environ.pop("MI355X_WG_TRACE_BUFFER", None)
-    for _ in range(warm_launches):   # the shader clock needs a few hundred launches to come up
-        launch()
-    torch.cuda.synchronize()
+    # The shader clock comes up with the time the part has been busy, not with the number of launches: after 500
+    # launches of a 13 us kernel (7 ms) its loop still reads 2.0 GHz, after 100 ms 2.3-2.4 GHz.
+    deadline = time.perf_counter() + warm_seconds
+    while time.perf_counter() < deadline:
+        for _ in range(200):
+            launch()
+        torch.cuda.synchronize()
     buf = torch.zeros(WORDS * max_workgroups, dtype=torch.int64, device="cuda")
     os.environ["MI355X_WG_TRACE_BUFFER"] = str(buf.data_ptr())
     os.environ["MI355X_WG_TRACE_CAPACITY"] = str(max_workgroups)   # workgroups beyond it write no stamps

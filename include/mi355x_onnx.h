@@ -58,7 +58,7 @@ int mi355x_device_cu_count(void);
 int mi355x_launch_empty_kernel(void* stream);
 
 /* The MI355X_* environment variables that force a kernel variant (MI355X_GEMM_CONFIG, MI355X_GEMM_NT_BN,
- * MI355X_GEMM_NT_BM, MI355X_GEMM_NT_BK, MI355X_GEMM_NT_PER_CU, MI355X_GEMM_GROUP_M, MI355X_GEMM_KSPLIT, MI355X_CONV_CONFIG, MI355X_CONV_GATHER_BN, MI355X_CONV_PER_CU, MI355X_CONV_TAIL, MI355X_CONV_STATIC_TAPS, MI355X_MMI_GENERIC,
+ * MI355X_GEMM_NT_BM, MI355X_GEMM_NT_BK, MI355X_GEMM_NT_PER_CU, MI355X_GEMM_NT_WAVES, MI355X_GEMM_GROUP_M, MI355X_GEMM_KSPLIT, MI355X_CONV_CONFIG, MI355X_CONV_GATHER_BN, MI355X_CONV_PER_CU, MI355X_CONV_TAIL, MI355X_CONV_STATIC_TAPS, MI355X_MMI_GENERIC,
  * MI355X_MMI_WGS_PER_CU, MI355X_MMI_TILE, MI355X_ATTN_WAVES) are read on the first launch only; call this after changing them. The role of
  * CudnnConvolution.default_algorithm / node._algorithm in the reference (cudnn_implementations.py:119-131):
  * a way to pick the algorithm by hand. */
