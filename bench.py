@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0
 # L2 <-> fabric bytes of the four GEMM launches of one layer, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script scaled by a copy kernel of known size (profiles/bert_layer_gemm_traffic.txt); counters cannot be
 # read from inside the process, so the figure is carried here and re-measured whenever the GEMM kernels change
-GEMM_TRAFFIC_BYTES_PER_LAYER = 175994604
+GEMM_TRAFFIC_BYTES_PER_LAYER = 176060019
 GEMM_TRAFFIC_SOURCE = "profiles/bert_layer_gemm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script; not re-measured by this run)"
 
 
