@@ -364,6 +364,9 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
     else if (best == 0) hipLaunchKernelGGL((gemm_f32_nt_kernel<3, 4, 2>), grid, block, 0, stream, p);
     else if (best == 1 && bk64 && p.K >= 2048) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2, 64, 3>), grid, block, 0, stream, p);  // 2.5 % at K = 3072, nothing at 1024
     else if (best == 1) hipLaunchKernelGGL((gemm_f32_nt_kernel<4, 4, 2>), grid, block, 0, stream, p);
+    // (128 x 96 tiles, one workgroup per CU, are never the library's own choice any more; as 16 waves, 8 wave rows x 2 k-split
+    // groups, they take 40.7 against 42.9 us on 1024 x 3072 x 768 and 288 against 302 us on 4096 x 4096 x 1024)
+    else if (best == 2 && tune.gemm_nt_waves != 8) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 2, 32, 3, 1>), grid, block16, 0, stream, p);
     else if (best == 2) hipLaunchKernelGGL((gemm_f32_nt_kernel<6, 8, 1>), grid, block, 0, stream, p);
     // the same for 128 x 48 tiles (80 registers, three workgroups per CU): 1024 x 3072 x 768 with Gelu takes 40.0 against
     // 42.2 us, 4096 x 4096 x 1024 246 against 262 us. Measured over 3072-wide outputs of 512 to 3328 tiles and K from 768

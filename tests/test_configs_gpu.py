@@ -275,7 +275,7 @@ def test_strided_gemm_head_split_merge_without_copies():
 
 
 # ----------------------------------------------------------------------------- GEMM kernel variants, ragged shapes
-@pytest.mark.parametrize("tile", ["auto", "48", "48x3", "48x2", "48w16", "64", "96", "144", "128x48", "128x48x3", "ksplit"])
+@pytest.mark.parametrize("tile", ["auto", "48", "48x3", "48x2", "48w16", "64", "96", "96w8", "144", "128x48", "128x48x3", "ksplit"])
 @pytest.mark.parametrize("M, N, K, epi", [(64, 48, 32, 0), (1, 4, 32, 1), (130, 52, 64, 9), (257, 100, 96, 5), (200, 148, 160, 3),
                                           (1024, 768, 768, 9), (63, 764, 224, 8), (100, 52, 2112, 9)])   # last: 64-k tiles
 def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
@@ -287,6 +287,8 @@ def test_k_contiguous_gemm_tiles_and_epilogues(tuning, tile, M, N, K, epi):
         tuning(MI355X_GEMM_NT_BM=128, MI355X_GEMM_NT_BN=48, MI355X_GEMM_NT_PER_CU=2)
     elif tile == "128x48x3":
         tuning(MI355X_GEMM_NT_BM=128, MI355X_GEMM_NT_BN=48, MI355X_GEMM_NT_PER_CU=3)
+    elif tile == "96w8":    # 128 x 96 tiles by eight waves (the library runs them as 16: 8 wave rows x 2 k-split groups)
+        tuning(MI355X_GEMM_NT_BN=96, MI355X_GEMM_NT_WAVES=8)
     elif tile == "48w16":   # 64 x 48 tiles by 16 waves, four k-split groups (where K is a multiple of 64; eight waves elsewhere)
         tuning(MI355X_GEMM_NT_BN=48, MI355X_GEMM_NT_WAVES=16)
     elif tile in ("48x3", "48x2"):   # 64 x 48 tiles as the lean kernel (three workgroups per CU) and as the 64-k one, whatever K
