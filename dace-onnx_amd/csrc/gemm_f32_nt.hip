@@ -318,6 +318,9 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
         double cost = (double)ceil_div(nwg, (int64_t)cus * cands[c].per_cu) * cands[c].per_cu * cands[c].bm * cands[c].bn * cands[c].weight;
         // (128 x 48 also runs three to a CU, in its lean form, 5 % faster per tile at full occupancy)
         if (c == 4) cost = std::min(cost, (double)ceil_div(nwg, (int64_t)cus * 3) * 3 * cands[c].bm * cands[c].bn * 0.74);
+        // (64 x 64 tiles have no lean form: over a short K their six-tile ring is most of the work before the first MFMA.
+        // 384 x 4096 x 256: 15.1 us against 13.5 us as 64 x 48; 1024 x 1024 x 256 stays with them, 8.7 against 10.5 us)
+        if (c == 1 && p.K <= 512) cost *= 1.15;
         if (force) {   // MI355X_GEMM_NT_BN picks the tile width, MI355X_GEMM_NT_BM the height where two candidates share a width
             if (force == cands[c].bn && (force_bm ? force_bm == cands[c].bm : cands[c].bm == 64 || cands[c].bn == 96)) { best = c; break; }
         } else if (cost < best_cost) {
