@@ -321,6 +321,10 @@ bool launch_gemm_f32_nt(GemmArgs p, int cus, hipStream_t stream) {
         // (64 x 64 tiles have no lean form: over a short K their six-tile ring is most of the work before the first MFMA.
         // 384 x 4096 x 256: 15.1 us against 13.5 us as 64 x 48; 1024 x 1024 x 256 stays with them, 8.7 against 10.5 us)
         if (c == 1 && p.K <= 512) cost *= 1.15;
+        // (128 x 96 tiles, 16 waves, one workgroup per CU: over a long K and in whole rounds -- where nothing of a round is
+        // wasted on them -- they are the fastest form by 1-3 %: 2048 x 3072 x 3072 270.9 against 280.3 us, 5120 x 3072 x 3072
+        // 671.8 against 691.1 us; with a ragged last round they lose by up to 10 %)
+        if (c == 2 && p.K >= 1536 && nwg % cus == 0) cost *= 0.75 / 0.8;
         if (force) {   // MI355X_GEMM_NT_BN picks the tile width, MI355X_GEMM_NT_BM the height where two candidates share a width
             if (force == cands[c].bn && (force_bm ? force_bm == cands[c].bm : cands[c].bm == 64 || cands[c].bn == 96)) { best = c; break; }
         } else if (cost < best_cost) {
